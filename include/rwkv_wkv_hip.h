@@ -1,0 +1,138 @@
+/*
+ * rwkv_wkv_hip -- C ABI of the MI355X (gfx950) WKV time-mix operators.
+ *
+ * One shared library, plain pointers and sizes, no framework types.  Every
+ * pointer is a DEVICE pointer unless stated; every call is asynchronous on the
+ * HIP stream passed in (a hipStream_t cast to void*; NULL = the default
+ * stream), allocates nothing and returns 0 or a negative wkv_status.
+ *
+ * Layouts (all contiguous, row-major):
+ *   r, k, v, y, gy, gr, gk, gv   (B, T, C) in `dtype`          C = H * 64
+ *   w (WKV6), gw (WKV6)          (B, T, C) fp32, RAW decay parameter:
+ *                                the decay applied is exp(-exp(w))
+ *   w (WKV5), gw (WKV5), u, gu   (H, 64)   fp32 (gw, gu summed over batch and time)
+ *   state                        (B, H, 64, 64) fp32, [key index][value index]
+ *   WKV4: time_decay, time_first (C) fp32;  state (B, C, 3) fp32 = (aa, bb, pp)
+ *
+ * Reference interfaces these entry points stand in for are cited per function
+ * (paths relative to the RWKV-infctx-trainer tree).
+ */
+#ifndef RWKV_WKV_HIP_H
+#define RWKV_WKV_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    WKV_OK = 0,
+    WKV_ERR_DIMS = -1,        /* non-positive size, C != H*64, T too large for 32-bit indexing */
+    WKV_ERR_NULL = -2,        /* a required pointer is NULL */
+    WKV_ERR_DTYPE = -3,       /* dtype not one of wkv_dtype */
+    WKV_ERR_ALIGN = -4,       /* a pointer is not 16-byte aligned */
+    WKV_ERR_WORKSPACE = -5,   /* workspace smaller than the matching *_workspace() query */
+    WKV_ERR_LAUNCH = -6,      /* HIP reported an error at launch */
+    WKV_ERR_ALGO = -7         /* algorithm not available for this shape / dtype */
+} wkv_status;
+
+typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
+
+/* flags */
+#define WKV_FLOOR_DECAY 1u    /* bound the decay below by 0.005 as the reference's chunked
+                                 training path does (RWKV-v5/src/module/rwkv_inner.py:40,48);
+                                 the gradient w.r.t. a floored w is zero */
+
+/* algorithm selector */
+#define WKV_ALGO_AUTO      0  /* chunked where it applies, else recurrent */
+#define WKV_ALGO_RECURRENT 1  /* per-token fp32 recurrence, any T, any dtype */
+#define WKV_ALGO_CHUNKED   2  /* 64-token chunks on the matrix cores, bf16 operands */
+
+const char *wkv_strerror(int status);
+int wkv_abi_version(void);
+
+/* ---------------------------------------------------------------- WKV6 ----
+ * Replaces wkv6state_cuda forward/backward as bound in
+ * RWKV-v6/src/module/cuda/wkv6state_op.cpp:5-17 and called from
+ * RWKV-v6/src/module/TimeMix.py:59-64,95-100; results follow the pure path
+ * RWKV-v6/src/module/rwkv_inner.py:10-115 (state in, state out, fp32 state,
+ * full state gradient).
+ */
+size_t wkv6_forward_workspace(int B, int T, int C, int H, int dtype, int algo);
+int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
+                 const void *r, const void *k, const void *v, const float *w, const float *u,
+                 const float *state_in, void *y, float *state_out,
+                 void *workspace, size_t workspace_bytes);
+
+size_t wkv6_backward_workspace(int B, int T, int C, int H, int dtype, int algo);
+/* gstate_out may be NULL (no gradient arrives through the state handed out,
+ * i.e. truncated BPTT); gstate_in may be NULL when it is not wanted. */
+int wkv6_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
+                  const void *r, const void *k, const void *v, const float *w, const float *u,
+                  const float *state_in, const void *gy, const float *gstate_out,
+                  void *gr, void *gk, void *gv, float *gw, float *gu, float *gstate_in,
+                  void *workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------- WKV5 ----
+ * Replaces wkv5 forward_{bf16,fp16,fp32} / backward_* of
+ * RWKV-v5/src/module/cuda/wkv5_op.cpp:84-129 (called from
+ * RWKV-v5/src/module/TimeMix.py:79-86,119-126); results follow
+ * RWKV-v5/src/module/rwkv_inner.py:10-118.  w, gw are per channel (H,64).
+ */
+size_t wkv5_forward_workspace(int B, int T, int C, int H, int dtype, int algo);
+int wkv5_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
+                 const void *r, const void *k, const void *v, const float *w, const float *u,
+                 const float *state_in, void *y, float *state_out,
+                 void *workspace, size_t workspace_bytes);
+
+size_t wkv5_backward_workspace(int B, int T, int C, int H, int dtype, int algo);
+int wkv5_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
+                  const void *r, const void *k, const void *v, const float *w, const float *u,
+                  const float *state_in, const void *gy, const float *gstate_out,
+                  void *gr, void *gk, void *gv, float *gw, float *gu, float *gstate_in,
+                  void *workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------- WKV4 ----
+ * Replaces cuda_forward / cuda_backward of
+ * RWKV-v4neo/cuda/wkv_cuda_bf16.cu:160-172 as wrapped by
+ * RWKV-v4neo/cuda/wkv_op_bf16.cpp:15-86 (torch.ops.rwkv.wkv).  time_decay is
+ * the RAW parameter (w = -exp(time_decay) is formed inside, as :34 does);
+ * g_time_decay, g_time_first are summed over the batch (as :85 does).
+ * state_in NULL means the empty history (0, 0, -1e38).  The state gradient is
+ * carried as (gp, gq, go) with go an exponent, as the reference does
+ * (wkv_cuda_bf16.cu:116-152).
+ * `checkpoints` (optional, wkv4_checkpoint_bytes() bytes): written by forward,
+ * read by backward, saves backward one sweep over k and v.
+ */
+size_t wkv4_checkpoint_bytes(int B, int T, int C);
+int wkv4_forward(void *stream, int B, int T, int C, int dtype,
+                 const float *time_decay, const float *time_first, const void *k, const void *v,
+                 const float *state_in, void *y, float *state_out, void *checkpoints);
+size_t wkv4_backward_workspace(int B, int T, int C, int dtype);
+int wkv4_backward(void *stream, int B, int T, int C, int dtype,
+                  const float *time_decay, const float *time_first, const void *k, const void *v,
+                  const float *state_in, const void *gy, const float *gstate_out,
+                  float *g_time_decay, float *g_time_first, void *gk, void *gv, float *gstate_in,
+                  const void *checkpoints, void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------ cumsum-decay ------
+ * The helper the reference's chunked path computes inline
+ * (RWKV-v5/src/module/rwkv_inner.py:43-58,72-79): from the raw decay parameter
+ * w (B,T,C) [or (1,1,C) broadcast when per_token == 0] to
+ *   log_w      (Bw,T,C)  max(-exp(w), ln 0.005)
+ *   incl       (Bw,T,C)  inclusive cumulative sum of log_w inside each chunk
+ *   inter      (Bw,T,C)  chunk total - incl   (decay from a token to its chunk's end)
+ *   intra      (Bw,T,C)  incl - log_w         (decay from the chunk's start to a token)
+ *   chunk_sum  (Bw,T/chunk,C)
+ * all fp32, in log space.  Any output pointer may be NULL.  T must be a
+ * multiple of chunk_len.
+ */
+int wkv_cumsum_decay(void *stream, int Bw, int T, int C, int chunk_len, int per_token,
+                     const float *w, float *log_w, float *incl, float *inter, float *intra,
+                     float *chunk_sum);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,180 @@
+// C ABI of the library: argument checks and dispatch.  This is the one
+// translation unit hipcc builds; the kernel files are included so that every
+// kernel and its launcher sit in the same code object.
+#include "../../include/rwkv_wkv_hip.h"
+#include "common.h"
+#include "wkv56_recurrent.hip"
+#include "wkv4.hip"
+#include "cumsum_decay.hip"
+
+using namespace wkv;
+
+namespace {
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_dims56(int B, int T, int C, int H, int dtype) {
+    if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return WKV_ERR_DIMS;
+    if (C != H * HEAD) return WKV_ERR_DIMS;
+    if ((long long)B * T * C >= (1ll << 40)) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    return WKV_OK;
+}
+
+int pick_algo56(int algo, int T, int dtype) {
+    if (algo == WKV_ALGO_AUTO) return WKV_ALGO_RECURRENT;
+    if (algo == WKV_ALGO_RECURRENT) return algo;
+    return WKV_ERR_ALGO;
+}
+
+int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
+              const void *r, const void *k, const void *v, const float *w, const float *u, const float *state_in,
+              void *y, float *state_out, void *workspace, size_t workspace_bytes) {
+    int st = check_dims56(B, T, C, H, dtype);
+    if (st) return st;
+    if (!r || !k || !v || !w || !u || !state_in || !y || !state_out) return WKV_ERR_NULL;
+    for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
+                          (const void *)state_out})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    const int a = pick_algo56(algo, T, dtype);
+    if (a < 0) return a;
+    (void)workspace; (void)workspace_bytes;
+    hipError_t e = recurrent_forward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
+                                     state_out, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+size_t backward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
+    if (check_dims56(B, T, C, H, dtype)) return 0;
+    return recurrent_backward_workspace(B, T, C);
+}
+
+int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
+               const void *r, const void *k, const void *v, const float *w, const float *u, const float *state_in,
+               const void *gy, const float *gstate_out, void *gr, void *gk, void *gv, float *gw, float *gu,
+               float *gstate_in, void *workspace, size_t workspace_bytes) {
+    int st = check_dims56(B, T, C, H, dtype);
+    if (st) return st;
+    if (!r || !k || !v || !w || !u || !state_in || !gy || !gr || !gk || !gv || !gw || !gu) return WKV_ERR_NULL;
+    for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, gy,
+                          (const void *)gstate_out, (const void *)gr, (const void *)gk, (const void *)gv,
+                          (const void *)gw, (const void *)gu, (const void *)gstate_in, (const void *)workspace})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    const int a = pick_algo56(algo, T, dtype);
+    if (a < 0) return a;
+    if (!workspace) return WKV_ERR_NULL;
+    if (workspace_bytes < backward56_workspace(B, T, C, H, dtype, algo)) return WKV_ERR_WORKSPACE;
+    hipError_t e = recurrent_backward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, gy,
+                                      gstate_out, gr, gk, gv, gw, gu, gstate_in, (float *)workspace,
+                                      (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int check_dims4(int B, int T, int C, int dtype) {
+    if (B <= 0 || T <= 0 || C <= 0) return WKV_ERR_DIMS;
+    if ((long long)B * C >= (1ll << 30)) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    return WKV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *wkv_strerror(int status) {
+    switch (status) {
+        case WKV_OK: return "ok";
+        case WKV_ERR_DIMS: return "bad dimensions (sizes must be positive and C == H*64)";
+        case WKV_ERR_NULL: return "a required pointer is NULL";
+        case WKV_ERR_DTYPE: return "unsupported dtype";
+        case WKV_ERR_ALIGN: return "pointer not 16-byte aligned";
+        case WKV_ERR_WORKSPACE: return "workspace too small";
+        case WKV_ERR_LAUNCH: return "HIP launch failed";
+        case WKV_ERR_ALGO: return "algorithm not available for this shape/dtype";
+        default: return "unknown status";
+    }
+}
+
+int wkv_abi_version(void) { return 1; }
+
+size_t wkv6_forward_workspace(int, int, int, int, int, int) { return 0; }
+size_t wkv5_forward_workspace(int, int, int, int, int, int) { return 0; }
+
+int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
+                 const void *k, const void *v, const float *w, const float *u, const float *state_in, void *y,
+                 float *state_out, void *workspace, size_t workspace_bytes) {
+    return forward56(true, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, y, state_out, workspace,
+                     workspace_bytes);
+}
+int wkv5_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
+                 const void *k, const void *v, const float *w, const float *u, const float *state_in, void *y,
+                 float *state_out, void *workspace, size_t workspace_bytes) {
+    return forward56(false, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, y, state_out, workspace,
+                     workspace_bytes);
+}
+
+size_t wkv6_backward_workspace(int B, int T, int C, int H, int dtype, int algo) {
+    return backward56_workspace(B, T, C, H, dtype, algo);
+}
+size_t wkv5_backward_workspace(int B, int T, int C, int H, int dtype, int algo) {
+    return backward56_workspace(B, T, C, H, dtype, algo);
+}
+
+int wkv6_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
+                  const void *k, const void *v, const float *w, const float *u, const float *state_in, const void *gy,
+                  const float *gstate_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gstate_in,
+                  void *workspace, size_t workspace_bytes) {
+    return backward56(true, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, gy, gstate_out, gr, gk, gv,
+                      gw, gu, gstate_in, workspace, workspace_bytes);
+}
+int wkv5_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
+                  const void *k, const void *v, const float *w, const float *u, const float *state_in, const void *gy,
+                  const float *gstate_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gstate_in,
+                  void *workspace, size_t workspace_bytes) {
+    return backward56(false, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, gy, gstate_out, gr, gk,
+                      gv, gw, gu, gstate_in, workspace, workspace_bytes);
+}
+
+size_t wkv4_checkpoint_bytes(int B, int T, int C) {
+    return (B > 0 && T > 0 && C > 0) ? v4_checkpoint_bytes(B, T, C) : 0;
+}
+size_t wkv4_backward_workspace(int B, int T, int C, int dtype) {
+    return check_dims4(B, T, C, dtype) ? 0 : v4_backward_workspace(B, T, C);
+}
+
+int wkv4_forward(void *stream, int B, int T, int C, int dtype, const float *time_decay, const float *time_first,
+                 const void *k, const void *v, const float *state_in, void *y, float *state_out, void *checkpoints) {
+    int st = check_dims4(B, T, C, dtype);
+    if (st) return st;
+    if (!time_decay || !time_first || !k || !v || !y) return WKV_ERR_NULL;
+    hipError_t e = v4_forward_dispatch((hipStream_t)stream, dtype, B, T, C, time_decay, time_first, k, v, state_in, y,
+                                       state_out, (float *)checkpoints);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv4_backward(void *stream, int B, int T, int C, int dtype, const float *time_decay, const float *time_first,
+                  const void *k, const void *v, const float *state_in, const void *gy, const float *gstate_out,
+                  float *g_time_decay, float *g_time_first, void *gk, void *gv, float *gstate_in,
+                  const void *checkpoints, void *workspace, size_t workspace_bytes) {
+    int st = check_dims4(B, T, C, dtype);
+    if (st) return st;
+    if (!time_decay || !time_first || !k || !v || !gy || !g_time_decay || !g_time_first || !gk || !gv || !workspace)
+        return WKV_ERR_NULL;
+    if (workspace_bytes < v4_backward_workspace(B, T, C)) return WKV_ERR_WORKSPACE;
+    hipError_t e = v4_backward_dispatch((hipStream_t)stream, dtype, B, T, C, time_decay, time_first, k, v, state_in, gy,
+                                        gstate_out, g_time_decay, g_time_first, gk, gv, gstate_in,
+                                        (const float *)checkpoints, (float *)workspace);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_cumsum_decay(void *stream, int Bw, int T, int C, int chunk_len, int per_token, const float *w, float *log_w,
+                     float *incl, float *inter, float *intra, float *chunk_sum) {
+    if (Bw <= 0 || T <= 0 || C <= 0 || chunk_len <= 0 || T % chunk_len != 0) return WKV_ERR_DIMS;
+    if (T / chunk_len > 65535 || Bw > 65535) return WKV_ERR_DIMS;
+    if (!w) return WKV_ERR_NULL;
+    hipError_t e = cumsum_decay_launch((hipStream_t)stream, Bw, T, C, chunk_len, per_token, w, log_w, incl, inter,
+                                       intra, chunk_sum);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -1,0 +1,77 @@
+// Shared device helpers: storage types, conversions, vector loads/stores.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace wkv {
+
+constexpr int HEAD = 64;                    // key size == value size of one head
+constexpr float LOG_W_FLOOR = -5.298317366548036f;   // ln 0.005
+
+struct bf16 { uint16_t bits; };
+struct f16 { _Float16 h; };
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16 x) { return __uint_as_float((uint32_t)x.bits << 16); }
+__device__ __forceinline__ float to_float(f16 x) { return (float)x.h; }
+
+__device__ __forceinline__ uint16_t bf16_bits(float f) {     // round to nearest even
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;     // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <class T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16 from_float<bf16>(float f) { return bf16{bf16_bits(f)}; }
+template <> __device__ __forceinline__ f16 from_float<f16>(float f) { return f16{(_Float16)f}; }
+
+// four consecutive elements <-> four floats (p must be aligned to 4 elements)
+__device__ __forceinline__ void load4(const float *p, float (&o)[4]) {
+    float4 x = *reinterpret_cast<const float4 *>(p);
+    o[0] = x.x; o[1] = x.y; o[2] = x.z; o[3] = x.w;
+}
+__device__ __forceinline__ void load4(const bf16 *p, float (&o)[4]) {
+    uint2 x = *reinterpret_cast<const uint2 *>(p);
+    o[0] = __uint_as_float(x.x << 16); o[1] = __uint_as_float(x.x & 0xffff0000u);
+    o[2] = __uint_as_float(x.y << 16); o[3] = __uint_as_float(x.y & 0xffff0000u);
+}
+__device__ __forceinline__ void load4(const f16 *p, float (&o)[4]) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    h4 x = *reinterpret_cast<const h4 *>(p);
+    o[0] = (float)x[0]; o[1] = (float)x[1]; o[2] = (float)x[2]; o[3] = (float)x[3];
+}
+__device__ __forceinline__ void store4(float *p, const float (&o)[4]) {
+    *reinterpret_cast<float4 *>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+__device__ __forceinline__ void store4(bf16 *p, const float (&o)[4]) {
+    uint2 x;
+    x.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+    x.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+    *reinterpret_cast<uint2 *>(p) = x;
+}
+__device__ __forceinline__ void store4(f16 *p, const float (&o)[4]) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    h4 x = {(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
+    *reinterpret_cast<h4 *>(p) = x;
+}
+
+// log of the decay from the raw parameter: -exp(x), optionally bounded below
+__device__ __forceinline__ float log_decay(float x, bool floor_decay, bool *floored = nullptr) {
+    float l = -__expf(x);
+    bool f = floor_decay && (l < LOG_W_FLOOR);
+    if (floored) *floored = f;
+    return f ? LOG_W_FLOOR : l;
+}
+
+// sum per-batch partials: in (B, n) -> out (n); fixed order, so repeatable
+static __global__ void sum_over_batch(int B, int n, const float *__restrict__ in, float *__restrict__ out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    for (int b = 0; b < B; b++) s += in[(size_t)b * n + i];
+    out[i] = s;
+}
+
+}  // namespace wkv

@@ -1,0 +1,48 @@
+// Cumulative-decay helper: from the raw decay parameter to the log-space
+// tables of the chunked formulation (RWKV-v5/src/module/rwkv_inner.py:43-58,
+// 72-79), in one fused pass.  log w = max(-exp(raw), ln 0.005) needs no log().
+// One lane per (batch, chunk, channel); consecutive lanes are consecutive
+// channels, so every row of every table is read and written coalesced.
+#include "common.h"
+
+namespace wkv {
+
+__global__ __launch_bounds__(256) void cumsum_decay_kernel(int Bw, int Tlen, int C, int chunk, int per_token,
+        const float *__restrict__ w, float *__restrict__ log_w, float *__restrict__ incl,
+        float *__restrict__ inter, float *__restrict__ intra, float *__restrict__ chunk_sum)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int n = blockIdx.y, b = blockIdx.z, nchunk = Tlen / chunk;
+    const size_t row0 = ((size_t)b * Tlen + (size_t)n * chunk) * C + c;
+    const float fixed = per_token ? 0.f : log_decay(w[c], true);
+
+    float total = 0.f;
+    if (per_token) {
+        for (int t = 0; t < chunk; t++) total += log_decay(w[row0 + (size_t)t * C], true);
+    } else {
+        for (int t = 0; t < chunk; t++) total += fixed;
+    }
+    if (chunk_sum) chunk_sum[((size_t)b * nchunk + n) * C + c] = total;
+
+    float run = 0.f;
+    for (int t = 0; t < chunk; t++) {
+        const size_t o = row0 + (size_t)t * C;
+        const float l = per_token ? log_decay(w[o], true) : fixed;
+        run += l;
+        if (log_w) log_w[o] = l;
+        if (incl) incl[o] = run;
+        if (inter) inter[o] = total - run;
+        if (intra) intra[o] = run - l;
+    }
+}
+
+hipError_t cumsum_decay_launch(hipStream_t s, int Bw, int Tlen, int C, int chunk, int per_token, const float *w,
+                               float *log_w, float *incl, float *inter, float *intra, float *chunk_sum) {
+    dim3 grid((C + 255) / 256, Tlen / chunk, Bw);
+    hipLaunchKernelGGL(cumsum_decay_kernel, grid, dim3(256), 0, s, Bw, Tlen, C, chunk, per_token, w, log_w, incl, inter,
+                       intra, chunk_sum);
+    return hipGetLastError();
+}
+
+}  // namespace wkv

@@ -1,0 +1,213 @@
+// RWKV-v4 WKV with (aa, bb, pp) state: one lane per (batch, channel) chain.
+//
+// The chain is serial in time, so the kernels keep many independent loads in
+// flight per lane instead: a block of 16 tokens of k, v (and gy) is fetched
+// into registers while the previous block is consumed; consecutive lanes are
+// consecutive channels, so every load and store is a full coalesced row.
+//
+// State convention (RWKV-v4neo/cuda/wkv_cuda_bf16.cu:30-52): (p, q, o) with
+// p, q the decayed sums divided by e^{o}.  Backward carries the state gradient
+// the same way, (gp, gq, go), and returns the decay gradient with respect to
+// the raw time_decay parameter (:116-156).
+//
+// Backward never stores per-token intermediates for the whole sequence (the
+// reference keeps three T-long arrays per lane): the forward sweep leaves a
+// 5-float checkpoint (p, q, o, dp/dw, dq/dw) every 16 tokens, and the backward
+// sweep replays one 16-token block at a time from its checkpoint.
+#include "common.h"
+
+namespace wkv {
+
+constexpr int CK = 16;                 // tokens per checkpoint block
+constexpr float NEG_HUGE = -1e38f;
+
+struct Chain { float p, q, o, dp, dq; };
+
+// one token: output y and the pieces backward re-uses; advances the chain
+__device__ __forceinline__ float v4_step(Chain &s, float w, float u, float kk, float vv,
+                                         float &iden, float &cexp, float &hist_w) {
+    const float m = fmaxf(s.o, u + kk);
+    hist_w = __expf(s.o - m);
+    cexp = u + kk - m;
+    const float ec = __expf(cexp);
+    iden = __frcp_rn(hist_w * s.q + ec);
+    const float y = (hist_w * s.p + ec * vv) * iden;
+    const float m2 = fmaxf(w + s.o, kk);
+    const float dh = __expf(w + s.o - m2), dc = __expf(kk - m2);
+    s.dp = dh * (s.p + s.dp);
+    s.dq = dh * (s.q + s.dq);
+    s.p = fmaf(dh, s.p, dc * vv);
+    s.q = fmaf(dh, s.q, dc);
+    s.o = m2;
+    return y;
+}
+
+// Forward.  y == nullptr: only checkpoints / final state are produced.
+// ckpt layout: [block][5][B*C].
+template <class T>
+__global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
+        const float *__restrict__ time_first, const T *__restrict__ k, const T *__restrict__ v,
+        const float *__restrict__ s_in, T *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= BC) return;
+    const int b = idx / C, c = idx % C;
+    const float w = -__expf(time_decay[c]), u = time_first[c];
+    const size_t base = (size_t)b * Tlen * C + c;
+    Chain s{0.f, 0.f, NEG_HUGE, 0.f, 0.f};
+    if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
+
+    float ck[CK], cv[CK], nk[CK], nv[CK];
+    auto fetch = [&](int t0, float (&kk)[CK], float (&vv)[CK]) {
+#pragma unroll
+        for (int i = 0; i < CK; i++) {
+            const bool in = t0 + i < Tlen;
+            kk[i] = in ? to_float(k[base + (size_t)(t0 + i) * C]) : 0.f;
+            vv[i] = in ? to_float(v[base + (size_t)(t0 + i) * C]) : 0.f;
+        }
+    };
+    fetch(0, ck, cv);
+    for (int t0 = 0, blk = 0; t0 < Tlen; t0 += CK, blk++) {
+        if (t0 + CK < Tlen) fetch(t0 + CK, nk, nv);
+        if (ckpt) {
+            float *cp = ckpt + (size_t)blk * 5 * BC + idx;
+            cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
+        }
+#pragma unroll
+        for (int i = 0; i < CK; i++) {
+            if (t0 + i < Tlen) {
+                float iden, cexp, hw;
+                const float yy = v4_step(s, w, u, ck[i], cv[i], iden, cexp, hw);
+                if (y) y[base + (size_t)(t0 + i) * C] = from_float<T>(yy);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < CK; i++) { ck[i] = nk[i]; cv[i] = nv[i]; }
+    }
+    if (s_out) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
+}
+
+template <class T>
+__global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
+        const float *__restrict__ time_first, const T *__restrict__ k, const T *__restrict__ v,
+        const T *__restrict__ gy, const float *__restrict__ gs_out, const float *__restrict__ ckpt,
+        float *__restrict__ gw_part, float *__restrict__ gu_part, T *__restrict__ gk, T *__restrict__ gv,
+        float *__restrict__ gs_in)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= BC) return;
+    const int b = idx / C, c = idx % C;
+    const float w = -__expf(time_decay[c]), u = time_first[c];
+    const size_t base = (size_t)b * Tlen * C + c;
+
+    float gp = 0.f, gq = 0.f, go = NEG_HUGE, acc_w = 0.f, acc_u = 0.f;
+    const int nblk = (Tlen + CK - 1) / CK;
+    for (int blk = nblk - 1; blk >= 0; blk--) {
+        const int t0 = blk * CK;
+        float kk[CK], vv[CK], gg[CK], ys[CK], iden[CK], cexp[CK];
+#pragma unroll
+        for (int i = 0; i < CK; i++) {
+            const bool in = t0 + i < Tlen;
+            const size_t o = base + (size_t)(t0 + i) * C;
+            kk[i] = in ? to_float(k[o]) : 0.f;
+            vv[i] = in ? to_float(v[o]) : 0.f;
+            gg[i] = in ? to_float(gy[o]) : 0.f;
+        }
+        const float *cp = ckpt + (size_t)blk * 5 * BC + idx;
+        Chain s{cp[0], cp[BC], cp[2 * (size_t)BC], cp[3 * (size_t)BC], cp[4 * (size_t)BC]};
+        // replay the block forward
+#pragma unroll
+        for (int i = 0; i < CK; i++) {
+            if (t0 + i < Tlen) {
+                const float dp0 = s.dp, dq0 = s.dq;
+                float hw;
+                ys[i] = v4_step(s, w, u, kk[i], vv[i], iden[i], cexp[i], hw);
+                acc_w += gg[i] * (dp0 - dq0 * ys[i]) * iden[i] * hw;
+                acc_u += gg[i] * (vv[i] - ys[i]) * __expf(cexp[i]) * iden[i];
+            }
+        }
+        if (blk == nblk - 1 && gs_out) {       // gradient arriving through the state handed out
+            gp = gs_out[idx * 3]; gq = gs_out[idx * 3 + 1]; go = gs_out[idx * 3 + 2];
+            if (gp == 0.f && gq == 0.f) go = NEG_HUGE;
+            acc_w += (gp * s.dp + gq * s.dq) * __expf(s.o + go);
+        }
+        // and walk it backwards
+#pragma unroll
+        for (int i = CK - 1; i >= 0; i--) {
+            if (t0 + i < Tlen) {
+                const size_t o = base + (size_t)(t0 + i) * C;
+                const float direct = gg[i] * iden[i] * __expf(cexp[i]);
+                const float later = __expf(kk[i] + go);
+                gk[o] = from_float<T>(direct * (vv[i] - ys[i]) + later * (gp * vv[i] + gq));
+                gv[o] = from_float<T>(direct + later * gp);
+                const float hist = cexp[i] - kk[i] - u;
+                const float m = fmaxf(w + go, hist);
+                const float keep = __expf(w + go - m);
+                const float add = gg[i] * iden[i] * __expf(hist - m);
+                gp = fmaf(keep, gp, add);
+                gq = fmaf(keep, gq, -add * ys[i]);
+                go = m;
+            }
+        }
+    }
+    if (gs_in) { gs_in[idx * 3] = gp; gs_in[idx * 3 + 1] = gq; gs_in[idx * 3 + 2] = go; }
+    gw_part[idx] = acc_w * w;
+    gu_part[idx] = acc_u;
+}
+
+size_t v4_checkpoint_bytes(int B, int Tlen, int C) {
+    return (size_t)((Tlen + CK - 1) / CK) * 5 * (size_t)B * C * sizeof(float);
+}
+size_t v4_backward_workspace(int B, int Tlen, int C) {       // gw, gu partials + room for checkpoints
+    return 2 * (size_t)B * C * sizeof(float) + v4_checkpoint_bytes(B, Tlen, C);
+}
+
+template <class T>
+static hipError_t fwd(hipStream_t s, int B, int Tlen, int C, const float *td, const float *tf, const void *k,
+                      const void *v, const float *s_in, void *y, float *s_out, float *ckpt) {
+    const int BC = B * C;
+    hipLaunchKernelGGL((v4_forward<T>), dim3((BC + 63) / 64), dim3(64), 0, s, BC, Tlen, C, td, tf, (const T *)k,
+                       (const T *)v, s_in, (T *)y, s_out, ckpt);
+    return hipGetLastError();
+}
+
+template <class T>
+static hipError_t bwd(hipStream_t s, int B, int Tlen, int C, const float *td, const float *tf, const void *k,
+                      const void *v, const float *s_in, const void *gy, const float *gs_out, float *gtd, float *gtf,
+                      void *gk, void *gv, float *gs_in, const float *ckpt, float *ws) {
+    const int BC = B * C;
+    float *gw_part = ws, *gu_part = ws + BC, *own_ckpt = ws + 2 * (size_t)BC;
+    if (!ckpt) {           // no checkpoints from the forward call: make them now
+        hipError_t e = fwd<T>(s, B, Tlen, C, td, tf, k, v, s_in, nullptr, nullptr, own_ckpt);
+        if (e != hipSuccess) return e;
+        ckpt = own_ckpt;
+    }
+    hipLaunchKernelGGL((v4_backward<T>), dim3((BC + 63) / 64), dim3(64), 0, s, BC, Tlen, C, td, tf, (const T *)k,
+                       (const T *)v, (const T *)gy, gs_out, ckpt, gw_part, gu_part, (T *)gk, (T *)gv, gs_in);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gw_part, gtd);
+    hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gu_part, gtf);
+    return hipGetLastError();
+}
+
+hipError_t v4_forward_dispatch(hipStream_t s, int dtype, int B, int Tlen, int C, const float *td, const float *tf,
+                               const void *k, const void *v, const float *s_in, void *y, float *s_out, float *ckpt) {
+    switch (dtype) {
+        case 0: return fwd<float>(s, B, Tlen, C, td, tf, k, v, s_in, y, s_out, ckpt);
+        case 1: return fwd<bf16>(s, B, Tlen, C, td, tf, k, v, s_in, y, s_out, ckpt);
+        default: return fwd<f16>(s, B, Tlen, C, td, tf, k, v, s_in, y, s_out, ckpt);
+    }
+}
+
+hipError_t v4_backward_dispatch(hipStream_t s, int dtype, int B, int Tlen, int C, const float *td, const float *tf,
+                                const void *k, const void *v, const float *s_in, const void *gy, const float *gs_out,
+                                float *gtd, float *gtf, void *gk, void *gv, float *gs_in, const float *ckpt, float *ws) {
+    switch (dtype) {
+        case 0: return bwd<float>(s, B, Tlen, C, td, tf, k, v, s_in, gy, gs_out, gtd, gtf, gk, gv, gs_in, ckpt, ws);
+        case 1: return bwd<bf16>(s, B, Tlen, C, td, tf, k, v, s_in, gy, gs_out, gtd, gtf, gk, gv, gs_in, ckpt, ws);
+        default: return bwd<f16>(s, B, Tlen, C, td, tf, k, v, s_in, gy, gs_out, gtd, gtf, gk, gv, gs_in, ckpt, ws);
+    }
+}
+
+}  // namespace wkv

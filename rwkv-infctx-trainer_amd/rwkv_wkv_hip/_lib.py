@@ -1,0 +1,69 @@
+"""ctypes binding of librwkv_wkv_hip.so (the C ABI declared in include/rwkv_wkv_hip.h).
+
+The library is prebuilt in-tree by ``make -C rwkv-infctx-trainer_amd/csrc`` (or
+``__graft_entry__.build()``).  There is no fallback: if it is missing, loading
+raises."""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_size_t, c_uint, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librwkv_wkv_hip.so")
+
+WKV_F32, WKV_BF16, WKV_F16 = 0, 1, 2
+FLOOR_DECAY = 1
+ALGO_AUTO, ALGO_RECURRENT, ALGO_CHUNKED = 0, 1, 2
+
+_P = c_void_p
+_I = c_int
+
+# name -> (restype, argtypes); the one list the symbol-export test walks
+SIGNATURES = {
+    "wkv_strerror": (c_char_p, [_I]),
+    "wkv_abi_version": (_I, []),
+    "wkv6_forward_workspace": (c_size_t, [_I] * 6),
+    "wkv6_forward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 8 + [_P, c_size_t]),
+    "wkv6_backward_workspace": (c_size_t, [_I] * 6),
+    "wkv6_backward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 14 + [_P, c_size_t]),
+    "wkv5_forward_workspace": (c_size_t, [_I] * 6),
+    "wkv5_forward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 8 + [_P, c_size_t]),
+    "wkv5_backward_workspace": (c_size_t, [_I] * 6),
+    "wkv5_backward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 14 + [_P, c_size_t]),
+    "wkv4_checkpoint_bytes": (c_size_t, [_I] * 3),
+    "wkv4_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 8),
+    "wkv4_backward_workspace": (c_size_t, [_I] * 4),
+    "wkv4_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, c_size_t]),
+    "wkv_cumsum_decay": (_I, [_P, _I, _I, _I, _I, _I] + [_P] * 6),
+}
+
+_lib = None
+
+
+class WKVError(RuntimeError):
+    pass
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise WKVError(
+                f"{LIB_PATH} is missing: build the HIP library first "
+                "(make -C rwkv-infctx-trainer_amd/csrc).  There is no CPU fallback.")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(status: int, what: str):
+    if status != 0:
+        msg = lib().wkv_strerror(status).decode()
+        if status in (-1, -3):
+            raise ValueError(f"{what}: {msg}")
+        raise WKVError(f"{what}: {msg} (status {status})")

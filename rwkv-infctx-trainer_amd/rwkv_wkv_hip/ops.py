@@ -1,0 +1,240 @@
+"""torch.autograd front ends with the reference trainer's call signatures.
+
+WKV_5.apply(B, T, C, H, state, r, k, v, w, u)  -> (y, new_state)
+WKV_6.apply(B, T, C, H, r, k, v, w, u, s)      -> (y, new_state)
+wkv_op(time_decay, time_first, k, v, wkv_state) -> (y, new_state)
+
+Argument order and meaning are those of WKV5_CUDA / WKV6STATE_CUDA
+(RWKV-v5/src/module/TimeMix.py:20-31, RWKV-v6/src/module/TimeMix.py:19-26) and
+of torch.ops.rwkv.wkv (RWKV-v4neo/src/model.py:130-132): ``w`` is the RAW decay
+parameter and the gradient returned for it is with respect to that raw
+parameter.  Unlike the reference's kernels the functions are functional (the
+new state is returned, and is differentiable); RUN_WKV5_CUDA /
+RUN_WKV6STATE_CUDA keep the reference's in-place convention on top of them.
+
+All tensors must live on the GPU; the work is done by librwkv_wkv_hip.so on the
+current HIP stream.
+"""
+from __future__ import annotations
+
+import os
+
+import torch
+
+from . import _lib
+from ._lib import WKVError, check
+
+HEAD = 64
+_DT = {torch.float32: _lib.WKV_F32, torch.bfloat16: _lib.WKV_BF16, torch.float16: _lib.WKV_F16}
+_ALGO = {"auto": _lib.ALGO_AUTO, "recurrent": _lib.ALGO_RECURRENT, "chunked": _lib.ALGO_CHUNKED}
+_algo = _ALGO[os.environ.get("RWKV_WKV_ALGO", "auto")]
+
+
+def set_algo(name: str):
+    """'auto' | 'recurrent' | 'chunked' for the WKV5/WKV6 operators."""
+    global _algo
+    _algo = _ALGO[name]
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _on_gpu(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise WKVError("rwkv_wkv_hip operators need GPU tensors (there is no CPU path)")
+
+
+def _check_rkv(B, T, C, H, r, k, v):
+    dtype = r.dtype
+    if dtype not in _DT:
+        raise ValueError(f"Unsupported dtype {dtype} for WKV")
+    assert dtype == k.dtype and dtype == v.dtype
+    assert r.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert r.shape == (B, T, C) and k.shape == (B, T, C) and v.shape == (B, T, C)
+    return _DT[dtype]
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32):
+    L = _lib.lib()
+    dt = _check_rkv(B, T, C, H, r, k, v)
+    _on_gpu(r, k, v, w32, u32, s32)
+    y = torch.empty_like(r)
+    new_state = torch.empty_like(s32)
+    flags = _lib.FLOOR_DECAY if T > 1 else 0
+    fn, wsq = (L.wkv5_forward, L.wkv5_forward_workspace) if version == 5 else (L.wkv6_forward, L.wkv6_forward_workspace)
+    nws = wsq(B, T, C, H, dt, _algo)
+    ws = _workspace(nws, r.device)
+    check(fn(_stream(), B, T, C, H, dt, flags, _algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
+             _ptr(y), _ptr(new_state), _ptr(ws), ws.numel()), f"wkv{version}_forward")
+    return y, new_state
+
+
+def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate):
+    L = _lib.lib()
+    dt = _DT[r.dtype]
+    gr, gk, gv = torch.empty_like(r), torch.empty_like(k), torch.empty_like(v)
+    gw = torch.empty_like(w32)
+    gu = torch.empty_like(u32)
+    gs = torch.empty_like(s32)
+    flags = _lib.FLOOR_DECAY if T > 1 else 0
+    fn, wsq = (L.wkv5_backward, L.wkv5_backward_workspace) if version == 5 else (L.wkv6_backward, L.wkv6_backward_workspace)
+    ws = _workspace(wsq(B, T, C, H, dt, _algo), r.device)
+    check(fn(_stream(), B, T, C, H, dt, flags, _algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
+             _ptr(gy), _ptr(gstate), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs), _ptr(ws), ws.numel()),
+          f"wkv{version}_backward")
+    return gr, gk, gv, gw, gu, gs
+
+
+class WKV_5(torch.autograd.Function):
+    """WKV5: per-channel decay.  state (B,H,64,64) fp32 [key][value]; r,k,v
+    (B,T,C) in one dtype; w (H,64) fp32 raw; u (H,64)."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, state, r, k, v, w, u):
+        assert state.dtype == torch.float32 and w.dtype == torch.float32
+        assert state.is_contiguous() and w.is_contiguous() and u.is_contiguous()
+        assert state.shape == (B, H, HEAD, HEAD) and H * HEAD == C
+        u32 = u.float().contiguous().view(H, HEAD)
+        w32 = w.view(H, HEAD)
+        with torch.no_grad():
+            y, new_state = _forward56(5, B, T, C, H, r, k, v, w32, u32, state)
+        ctx.dims = (B, T, C, H)
+        ctx.meta = (w.shape, u.shape, u.dtype)
+        ctx.save_for_backward(r, k, v, w32, u32, state)
+        return y, new_state
+
+    @staticmethod
+    def backward(ctx, gy, gstate):
+        B, T, C, H = ctx.dims
+        r, k, v, w32, u32, state = ctx.saved_tensors
+        wshape, ushape, udtype = ctx.meta
+        gy = gy.contiguous()
+        assert gy.dtype == r.dtype
+        gstate = None if gstate is None else gstate.float().contiguous()
+        with torch.no_grad():
+            gr, gk, gv, gw, gu, gs = _backward56(5, B, T, C, H, r, k, v, w32, u32, state, gy, gstate)
+        return (None, None, None, None, gs, gr, gk, gv, gw.view(wshape), gu.view(ushape).to(udtype))
+
+
+class WKV_6(torch.autograd.Function):
+    """WKV6: per-token decay.  r,k,v (B,T,C); w (B,T,C) raw (any float dtype,
+    used in fp32); u (H,64); s (B,H,64,64) [key][value]."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u, s):
+        assert s.is_contiguous() and w.is_contiguous() and u.is_contiguous()
+        assert s.shape == (B, H, HEAD, HEAD) and H * HEAD == C and w.shape == (B, T, C)
+        u32 = u.float().contiguous().view(H, HEAD)
+        w32 = w.float()
+        s32 = s.float()
+        with torch.no_grad():
+            y, new_state = _forward56(6, B, T, C, H, r, k, v, w32, u32, s32)
+        ctx.dims = (B, T, C, H)
+        ctx.meta = (w.dtype, u.shape, u.dtype, s.dtype)
+        ctx.save_for_backward(r, k, v, w32, u32, s32)
+        return y, new_state.to(s.dtype)
+
+    @staticmethod
+    def backward(ctx, gy, gstate):
+        B, T, C, H = ctx.dims
+        r, k, v, w32, u32, s32 = ctx.saved_tensors
+        wdtype, ushape, udtype, sdtype = ctx.meta
+        gy = gy.contiguous()
+        assert gy.dtype == r.dtype
+        gstate = None if gstate is None else gstate.float().contiguous()
+        with torch.no_grad():
+            gr, gk, gv, gw, gu, gs = _backward56(6, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate)
+        return (None, None, None, None, gr, gk, gv, gw.to(wdtype), gu.view(ushape).to(udtype), gs.to(sdtype))
+
+
+def RUN_WKV5_CUDA(B, T, C, H, state, r, k, v, w, u):
+    """The reference's calling convention (RWKV-v5/src/module/TimeMix.py:145-154):
+    returns y and leaves the new state in ``state``."""
+    y, new_state = WKV_5.apply(B, T, C, H, state, r, k, v, w, u)
+    with torch.no_grad():
+        state.copy_(new_state)
+    return y
+
+
+def RUN_WKV6STATE_CUDA(B, T, C, H, r, k, v, w, u, s):
+    """The reference's calling convention (RWKV-v6/src/module/TimeMix.py:111-118):
+    returns y and leaves the new state in ``s``."""
+    y, new_state = WKV_6.apply(B, T, C, H, r, k, v, w, u, s)
+    with torch.no_grad():
+        s.copy_(new_state)
+    return y
+
+
+class _WKV4(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, time_decay, time_first, k, v, wkv_state):
+        L = _lib.lib()
+        assert k.dim() == 3 and v.shape == k.shape and k.dtype == v.dtype
+        B, T, C = k.shape
+        assert time_decay.shape == (C,) and time_first.shape == (C,) and wkv_state.shape == (B, C, 3)
+        if k.dtype not in _DT:
+            raise ValueError(f"Unsupported dtype {k.dtype} for WKV")
+        _on_gpu(time_decay, time_first, k, v, wkv_state)
+        td, tf = time_decay.float().contiguous(), time_first.float().contiguous()
+        k, v, st = k.contiguous(), v.contiguous(), wkv_state.float().contiguous()
+        y = torch.empty_like(k)
+        new_state = torch.empty_like(st)
+        need_grad = any(t.requires_grad for t in (time_decay, time_first, k, v, wkv_state))
+        ckpt = _workspace(L.wkv4_checkpoint_bytes(B, T, C), k.device) if need_grad else None
+        check(L.wkv4_forward(_stream(), B, T, C, _DT[k.dtype], _ptr(td), _ptr(tf), _ptr(k), _ptr(v), _ptr(st),
+                             _ptr(y), _ptr(new_state), _ptr(ckpt)), "wkv4_forward")
+        ctx.save_for_backward(td, tf, k, v, st, ckpt)
+        ctx.meta = (time_decay.dtype, time_first.dtype)
+        return y, new_state
+
+    @staticmethod
+    def backward(ctx, gy, gnew_state):
+        L = _lib.lib()
+        td, tf, k, v, st, ckpt = ctx.saved_tensors
+        B, T, C = k.shape
+        gy = gy.contiguous()
+        gns = None if gnew_state is None else gnew_state.float().contiguous()
+        gtd, gtf = torch.empty_like(td), torch.empty_like(tf)
+        gk, gv = torch.empty_like(k), torch.empty_like(v)
+        gst = torch.empty_like(st)
+        ws = _workspace(L.wkv4_backward_workspace(B, T, C, _DT[k.dtype]), k.device)
+        check(L.wkv4_backward(_stream(), B, T, C, _DT[k.dtype], _ptr(td), _ptr(tf), _ptr(k), _ptr(v), _ptr(st),
+                              _ptr(gy), _ptr(gns), _ptr(gtd), _ptr(gtf), _ptr(gk), _ptr(gv), _ptr(gst), _ptr(ckpt),
+                              _ptr(ws), ws.numel()), "wkv4_backward")
+        return gtd.to(ctx.meta[0]), gtf.to(ctx.meta[1]), gk, gv, gst
+
+
+def wkv_op(time_decay, time_first, k, v, wkv_state):
+    """RWKV-v4 WKV with the signature of torch.ops.rwkv.wkv
+    (RWKV-v4neo/src/model.py:130-132): time_decay, time_first (C); k, v (B,T,C);
+    wkv_state (B,C,3) = (aa, bb, pp).  Returns (y, new_state)."""
+    return _WKV4.apply(time_decay, time_first, k, v, wkv_state)
+
+
+def cumsum_decay(w, chunk_len=128, per_token=True):
+    """Log-space decay tables of the chunked formulation from the raw decay
+    parameter w (B,T,C) fp32, or (C,) expanded over T tokens when
+    ``per_token`` is an int T.  Returns dict(log_w, incl, inter, intra, chunk_sum)."""
+    L = _lib.lib()
+    _on_gpu(w)
+    w = w.float().contiguous()
+    if w.dim() == 3:
+        Bw, T, C = w.shape
+        pt = 1
+    else:
+        (C,), Bw, T, pt = w.shape, 1, int(per_token), 0
+    out = {n: torch.empty(Bw, T, C, dtype=torch.float32, device=w.device) for n in ("log_w", "incl", "inter", "intra")}
+    out["chunk_sum"] = torch.empty(Bw, T // chunk_len, C, dtype=torch.float32, device=w.device)
+    check(L.wkv_cumsum_decay(_stream(), Bw, T, C, chunk_len, pt, _ptr(w), _ptr(out["log_w"]), _ptr(out["incl"]),
+                             _ptr(out["inter"]), _ptr(out["intra"]), _ptr(out["chunk_sum"])), "wkv_cumsum_decay")
+    return out

@@ -1,0 +1,237 @@
+"""GPU parity: the HIP operators (through the C ABI and the autograd front
+ends) against the CPU oracle on identical seeded inputs.
+
+Tolerances (written where used): rtol 1e-3 for fp32 I/O, 2e-2 for bf16/fp16
+I/O, each with an absolute floor of rtol * rms(reference tensor).  The oracle
+runs in fp32 on the already-rounded inputs."""
+import pytest
+import torch
+
+from oracle import wkv4 as O4
+from oracle import wkv56 as O
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float32: 1e-3, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+NAMES = ("y", "state", "gr", "gk", "gv", "gw", "gu", "gstate")
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def run_gpu56(version, wl, with_gstate=True, algo="auto"):
+    import rwkv_wkv_hip as W
+    W.set_algo(algo)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.to(dev()) for n, x in wl.tensors.items()}
+    leaves = {n: g[n].clone().requires_grad_(True) for n in ("r", "k", "v", "w", "u", "state")}
+    if version == 5:
+        y, s = W.WKV_5.apply(B, T, C, H, leaves["state"], leaves["r"], leaves["k"], leaves["v"], leaves["w"], leaves["u"])
+    else:
+        y, s = W.WKV_6.apply(B, T, C, H, leaves["r"], leaves["k"], leaves["v"], leaves["w"], leaves["u"], leaves["state"])
+    if with_gstate:
+        torch.autograd.backward([y, s], [g["dy"], g["dstate"]])
+    else:
+        y.backward(g["dy"])
+    torch.cuda.synchronize()
+    W.set_algo("auto")
+    return dict(y=y, state=s, gr=leaves["r"].grad, gk=leaves["k"].grad, gv=leaves["v"].grad, gw=leaves["w"].grad,
+                gu=leaves["u"].grad, gstate=leaves["state"].grad)
+
+
+def run_oracle56(version, wl, with_gstate=True):
+    t = wl.tensors
+    gs = t["dstate"] if with_gstate else torch.zeros_like(t["dstate"])
+    return O.wkv_op_grads(version, wl.B, wl.T, wl.C, wl.H, t["r"].float(), t["k"].float(), t["v"].float(), t["w"],
+                          t["u"], t["state"], t["dy"].float(), gs)
+
+
+def compare(got, ref, rtol, tag):
+    for n in NAMES:
+        assert_close(got[n], ref[n], rtol, f"{tag}:{n}")
+
+
+@pytest.mark.parametrize("version", [5, 6])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T", [1, 7, 16, 17, 128, 200, 256])
+def test_recurrent_matches_oracle(version, dtype, T):
+    from rwkv_wkv_hip import configs
+    cfg = 1 if version == 5 else 3
+    wl = configs.make(cfg, B=2, T=T, C=128, H=2, dtype=dtype)
+    print(f"case v{version} {dtype} T={T}", flush=True)
+    got = run_gpu56(version, wl, algo="recurrent")
+    ref = run_oracle56(version, wl)
+    compare(got, ref, RTOL[dtype], f"v{version}/{dtype}/T{T}")
+
+
+@pytest.mark.parametrize("version", [5, 6])
+def test_floor_on_decay_and_its_zero_gradient(version):
+    """Raw decays large enough that exp(-exp(w)) < 0.005: the operator uses
+    0.005 and returns a zero gradient there, as the chunked reference path."""
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=1, T=128, C=64, H=1, dtype=torch.float32)
+    w = wl.tensors["w"]
+    if version == 5:
+        w[0, 3] = 2.5
+        w[0, 17] = 1.8
+    else:
+        w[0, 5, 3] = 2.5
+        w[0, 77, 40] = 4.0
+    got = run_gpu56(version, wl, algo="recurrent")
+    ref = run_oracle56(version, wl)
+    compare(got, ref, 1e-3, f"floor v{version}")
+    gw = got["gw"].cpu()
+    if version == 5:
+        assert gw[0, 3] == 0 and gw[0, 17] == 0 and gw[0, 4] != 0
+    else:
+        assert gw[0, 5, 3] == 0 and gw[0, 77, 40] == 0 and gw[0, 5, 4] != 0
+
+
+@pytest.mark.parametrize("version", [5, 6])
+def test_no_state_gradient_truncated_bptt(version):
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=2, T=128, C=128, H=2, dtype=torch.bfloat16)
+    got = run_gpu56(version, wl, with_gstate=False, algo="recurrent")
+    ref = run_oracle56(version, wl, with_gstate=False)
+    for n in NAMES:
+        assert_close(got[n], ref[n], 2e-2, f"trunc v{version}:{n}")
+
+
+def test_segment_chain_equals_one_call_v6():
+    """Two chained calls over T tokens each, with the state gradient handed
+    back, equal one call over 2T tokens (outputs and every gradient)."""
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import configs
+    W.set_algo("recurrent")
+    wl = configs.make(3, B=2, T=256, C=128, H=2, dtype=torch.float32)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.to(dev()) for n, x in wl.tensors.items()}
+    L1 = {n: g[n].clone().requires_grad_(True) for n in ("r", "k", "v", "w", "u", "state")}
+    y, s = W.WKV_6.apply(B, T, C, H, L1["r"], L1["k"], L1["v"], L1["w"], L1["u"], L1["state"])
+    torch.autograd.backward([y, s], [g["dy"], g["dstate"]])
+    L2 = {n: g[n].clone().requires_grad_(True) for n in ("r", "k", "v", "w", "u", "state")}
+    h = T // 2
+    a = lambda x: x[:, :h].contiguous()
+    b = lambda x: x[:, h:].contiguous()
+    y1, s1 = W.WKV_6.apply(B, h, C, H, a(L2["r"]), a(L2["k"]), a(L2["v"]), a(L2["w"]), L2["u"], L2["state"])
+    y2, s2 = W.WKV_6.apply(B, h, C, H, b(L2["r"]), b(L2["k"]), b(L2["v"]), b(L2["w"]), L2["u"], s1)
+    torch.autograd.backward([y1, y2, s2], [a(g["dy"]), b(g["dy"]), g["dstate"]])
+    torch.cuda.synchronize()
+    W.set_algo("auto")
+    assert_close(torch.cat([y1, y2], 1), y, 1e-5, "chain y")
+    assert_close(s2, s, 1e-5, "chain state")
+    for n in ("r", "k", "v", "w", "u", "state"):
+        assert_close(L2[n].grad, L1[n].grad, 1e-4, f"chain g{n}")
+
+
+def test_in_place_wrappers_keep_reference_convention():
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1, B=1, T=32, C=128, H=2, dtype=torch.bfloat16)
+    g = {n: x.to(dev()) for n, x in wl.tensors.items()}
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    st = g["state"].clone()
+    y = W.RUN_WKV5_CUDA(B, T, C, H, st, g["r"], g["k"], g["v"], g["w"], g["u"].to(torch.bfloat16))
+    y2, ns = W.WKV_5.apply(B, T, C, H, g["state"], g["r"], g["k"], g["v"], g["w"], g["u"])
+    assert y.shape == (B, T, C) and y.dtype == torch.bfloat16
+    assert torch.equal(st, ns) and not torch.equal(st, g["state"])
+    wl6 = configs.make(3, B=1, T=32, C=128, H=2, dtype=torch.bfloat16)
+    g6 = {n: x.to(dev()) for n, x in wl6.tensors.items()}
+    s6 = g6["state"].clone()
+    y6 = W.WKV6STATE_CUDA.apply(B, T, C, H, g6["r"], g6["k"], g6["v"], g6["w"], g6["u"], s6)
+    _, ns6 = W.WKV_6.apply(B, T, C, H, g6["r"], g6["k"], g6["v"], g6["w"], g6["u"], g6["state"])
+    assert torch.equal(s6, ns6) and y6.dtype == torch.bfloat16
+
+
+# ------------------------------------------------------------------ v4 -----
+def v4_case(B, T, C, dtype, seed=0, with_state=False):
+    from rwkv_wkv_hip import configs
+    wl = configs.make(2, B=B, T=T, C=C, dtype=dtype, seed=seed)
+    t = wl.tensors
+    if with_state:
+        g = torch.Generator().manual_seed(seed + 50)
+        t["state"] = torch.stack([torch.randn(B, C, generator=g), torch.rand(B, C, generator=g) + 0.5,
+                                  torch.randn(B, C, generator=g)], -1)
+        t["dstate"] = torch.stack([torch.randn(B, C, generator=g), torch.randn(B, C, generator=g),
+                                   torch.randn(B, C, generator=g) * 0.3], -1)
+    return wl
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,with_state", [(1, False), (16, False), (37, True), (128, True), (300, False)])
+def test_v4_matches_oracle(dtype, T, with_state):
+    import rwkv_wkv_hip as W
+    B, C = 3, 96
+    wl = v4_case(B, T, C, dtype, with_state=with_state)
+    t = wl.tensors
+    print(f"case v4 {dtype} T={T} state={with_state}", flush=True)
+    f32 = lambda x: x.float()
+    y_ref, s_ref = O4.forward(t["time_decay"], f32(t["time_first"]), f32(t["k"]), f32(t["v"]), t["state"])
+    ref = O4.backward(t["time_decay"], f32(t["time_first"]), f32(t["k"]), f32(t["v"]), t["state"], f32(t["dy"]),
+                      t["dstate"])
+    g = {n: x.to(dev()) for n, x in t.items()}
+    L = {n: g[n].clone().requires_grad_(True) for n in ("time_decay", "time_first", "k", "v", "state")}
+    y, s = W.wkv_op(L["time_decay"], L["time_first"], L["k"], L["v"], L["state"])
+    torch.autograd.backward([y, s], [g["dy"], g["dstate"]])
+    torch.cuda.synchronize()
+    rt = RTOL[dtype]
+    assert_close(y, y_ref, rt, "v4 y")
+    und = lambda st: st[..., :2].float().cpu() * torch.exp(st[..., 2:3].float().cpu())
+    assert_close(und(s), und(s_ref), 1e-3, "v4 state (undivided sums)")
+    assert_close(L["time_decay"].grad, ref[0], rt, "v4 g_time_decay")
+    assert_close(L["time_first"].grad, ref[1], rt, "v4 g_time_first")
+    assert_close(L["k"].grad, ref[2], rt, "v4 gk")
+    assert_close(L["v"].grad, ref[3], rt, "v4 gv")
+    assert_close(und(L["state"].grad), und(ref[4]), rt, "v4 gstate (undivided)")
+
+
+def test_v4_backward_without_forward_checkpoints():
+    """The C entry point rebuilds its checkpoints when none are passed."""
+    import ctypes
+    from rwkv_wkv_hip import _lib
+    L = _lib.lib()
+    B, T, C = 2, 50, 64
+    wl = v4_case(B, T, C, torch.float32, seed=3, with_state=True)
+    t = wl.tensors
+    ref = O4.backward(t["time_decay"], t["time_first"], t["k"], t["v"], t["state"], t["dy"], t["dstate"])
+    g = {n: x.to(dev()).contiguous() for n, x in t.items()}
+    gtd, gtf = torch.empty(C, device=dev()), torch.empty(C, device=dev())
+    gk, gv, gst = torch.empty_like(g["k"]), torch.empty_like(g["v"]), torch.empty_like(g["state"])
+    ws = torch.empty(L.wkv4_backward_workspace(B, T, C, 0), dtype=torch.uint8, device=dev())
+    p = lambda x: x.data_ptr()
+    st = L.wkv4_backward(None, B, T, C, 0, p(g["time_decay"]), p(g["time_first"]), p(g["k"]), p(g["v"]), p(g["state"]),
+                         p(g["dy"]), p(g["dstate"]), p(gtd), p(gtf), p(gk), p(gv), p(gst), None, p(ws), ws.numel())
+    torch.cuda.synchronize()
+    assert st == 0
+    assert_close(gk, ref[2], 1e-3, "gk")
+    assert_close(gv, ref[3], 1e-3, "gv")
+    assert_close(gtd, ref[0], 1e-3, "gtd")
+
+
+# -------------------------------------------------------------- helper -----
+@pytest.mark.parametrize("chunk", [16, 128])
+def test_cumsum_decay_helper(chunk):
+    import rwkv_wkv_hip as W
+    B, T, H, K = 2, 256, 3, 64
+    C = H * K
+    g = torch.Generator().manual_seed(11)
+    raw = torch.randn(B, T, C, generator=g) * 0.8 - 0.5
+    raw[0, 9, 5] = 3.0                                   # below the floor
+    out = W.cumsum_decay(raw.to(dev()), chunk)
+    w = O.decay_from_raw(raw).view(B, T, H, K).transpose(1, 2)           # (B,H,T,K)
+    tab = O.cumsum_decay(w, chunk, 64)
+    back = lambda x: x.reshape(B, H, T, K).transpose(1, 2).reshape(B, T, C)
+    assert_close(out["log_w"], back(tab.log_w), 1e-5, "log_w")
+    assert_close(out["incl"], back(tab.incl), 1e-5, "incl")
+    assert_close(out["inter"], back(tab.inter_log), 1e-5, "inter")
+    assert_close(out["intra"], back(tab.intra_log), 1e-5, "intra")
+    cs = tab.chunk_log[..., 0, :].transpose(1, 2).reshape(B, T // chunk, C)
+    assert_close(out["chunk_sum"], cs, 1e-5, "chunk_sum")
+    assert out["log_w"][0, 9, 5].item() == pytest.approx(-5.298317, abs=1e-5)
+    # per-channel (WKV5) form
+    out5 = W.cumsum_decay(raw[0, 0].to(dev()), chunk, per_token=T)
+    w5 = O.decay_from_raw(raw[0, 0]).view(1, H, 1, K).expand(1, H, T, K)
+    tab5 = O.cumsum_decay(w5, chunk, 64)
+    assert_close(out5["incl"], tab5.incl.reshape(1, H, T, K).transpose(1, 2).reshape(1, T, C), 1e-5, "incl v5")
