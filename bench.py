@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the WKV hot path on one MI355X.
+
+Default workload (``--cfg 4``): WKV6 forward+backward on one 4096-token BPTT
+segment at the RWKV-v6 7B layer shape (B=1, C=4096, H=64, head 64; bf16 r/k/v/dy,
+fp32 raw decay, fp32 state), the state carried from step to step and the state
+gradient fed back, i.e. one link of the long-context chain per step.  A "step"
+is one forward + one backward call through the C ABI with all inputs resident
+in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cfg 1|2|3|4] [--algo auto|recurrent|chunked]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "rwkv-infctx-trainer_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cfg", type=int, default=4, choices=[1, 2, 3, 4])
+    ap.add_argument("--algo", default="auto", choices=["auto", "recurrent", "chunked"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline times")
+    ap.add_argument("--rotate", type=int, default=3, help="distinct input sets cycled through")
+    return ap.parse_args()
+
+
+class Runner56:
+    """WKV5 / WKV6 forward+backward through the C ABI on preallocated buffers."""
+
+    def __init__(self, cfg, algo, rotate):
+        import torch
+        from rwkv_wkv_hip import _lib, configs
+        self.torch, self._lib, self.L = torch, _lib, _lib.lib()
+        dev = torch.device("cuda:0")
+        self.sets = []
+        for i in range(rotate):
+            wl = configs.make(cfg, seed=1000 + cfg + i)
+            self.sets.append({n: t.to(dev).contiguous() for n, t in wl.tensors.items()})
+        self.wl = wl
+        self.version = wl.version
+        B, T, C, H = wl.B, wl.T, wl.C, wl.H
+        self.dims = (B, T, C, H)
+        self.dt = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[wl.dtype]
+        self.algo = {"auto": 0, "recurrent": 1, "chunked": 2}[algo]
+        s0 = self.sets[0]
+        self.y, self.gr, self.gk, self.gv = (torch.empty_like(s0["r"]) for _ in range(4))
+        self.gw = torch.empty_like(s0["w"])
+        self.gu = torch.empty_like(s0["u"])
+        self.state = [s0["state"].clone(), torch.empty_like(s0["state"])]
+        self.gstate_in = torch.empty_like(s0["state"])
+        L = self.L
+        q = (L.wkv5_forward_workspace, L.wkv5_backward_workspace) if self.version == 5 else \
+            (L.wkv6_forward_workspace, L.wkv6_backward_workspace)
+        nws = max(q[0](B, T, C, H, self.dt, self.algo), q[1](B, T, C, H, self.dt, self.algo), 16)
+        self.ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+        self.fwd = L.wkv5_forward if self.version == 5 else L.wkv6_forward
+        self.bwd = L.wkv5_backward if self.version == 5 else L.wkv6_backward
+        self.stream = torch.cuda.current_stream().cuda_stream
+        self.i = 0
+        self.tokens_per_step = B * T
+        elems = B * T * C
+        st = B * H * 64 * 64 * 4
+        per = 34 if self.version == 6 else 22
+        self.bytes_step = per * elems + 5 * st
+        self.bytes_fwd = (12 if self.version == 6 else 8) * elems + 2 * st
+        self.bytes_bwd = (22 if self.version == 6 else 14) * elems + 3 * st
+        self.dtype_name = "bf16"
+        self.desc = (f"cfg{cfg}: WKV{self.version} fwd+bwd B{B} T{T} C{C} H{H} head 64, bf16 r/k/v/dy, fp32 "
+                     f"raw decay and state, state carried step to step, state gradient fed back")
+
+    def step(self):
+        B, T, C, H = self.dims
+        s = self.sets[self.i % len(self.sets)]
+        s_in, s_out = self.state[self.i % 2], self.state[(self.i + 1) % 2]
+        self.i += 1
+        p = lambda t: t.data_ptr()
+        flags = self._lib.FLOOR_DECAY
+        st = self.fwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
+                      p(s["u"]), p(s_in), p(self.y), p(s_out), p(self.ws), self.ws.numel())
+        assert st == 0, self.L.wkv_strerror(st)
+        st = self.bwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
+                      p(s["u"]), p(s_in), p(s["dy"]), p(s["dstate"]), p(self.gr), p(self.gk), p(self.gv), p(self.gw),
+                      p(self.gu), p(self.gstate_in), p(self.ws), self.ws.numel())
+        assert st == 0, self.L.wkv_strerror(st)
+
+    def kernel_ids(self):
+        return {"forward": (1, 10), "backward": (2, 11)}
+
+
+class Runner4:
+    """WKV4 forward+backward through the C ABI (cfg2)."""
+
+    def __init__(self, cfg, algo, rotate):
+        import torch
+        from rwkv_wkv_hip import _lib, configs
+        self.torch, self._lib, self.L = torch, _lib, _lib.lib()
+        dev = torch.device("cuda:0")
+        self.sets = []
+        for i in range(rotate):
+            wl = configs.make(cfg, seed=1000 + cfg + i)
+            self.sets.append({n: t.to(dev).contiguous() for n, t in wl.tensors.items()})
+        B, T, C = wl.B, wl.T, wl.C
+        self.dims = (B, T, C)
+        s0 = self.sets[0]
+        self.y, self.gk, self.gv = (torch.empty_like(s0["k"]) for _ in range(3))
+        self.gtd, self.gtf = torch.empty(C, device=dev), torch.empty(C, device=dev)
+        self.state = [s0["state"].clone(), torch.empty_like(s0["state"])]
+        self.gstate = torch.empty_like(s0["state"])
+        self.ckpt = torch.empty(self.L.wkv4_checkpoint_bytes(B, T, C), dtype=torch.uint8, device=dev)
+        self.ws = torch.empty(self.L.wkv4_backward_workspace(B, T, C, 0), dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.current_stream().cuda_stream
+        self.i = 0
+        self.tokens_per_step = B * T
+        elems = B * T * C
+        self.bytes_step, self.bytes_fwd, self.bytes_bwd = 32 * elems, 12 * elems, 20 * elems
+        self.dtype_name = "f32"
+        self.desc = f"cfg{cfg}: WKV4 fwd+bwd B{B} T{T} C{C} fp32, (aa,bb,pp) state carried step to step"
+
+    def step(self):
+        B, T, C = self.dims
+        s = self.sets[self.i % len(self.sets)]
+        s_in, s_out = self.state[self.i % 2], self.state[(self.i + 1) % 2]
+        self.i += 1
+        p = lambda t: t.data_ptr()
+        st = self.L.wkv4_forward(self.stream, B, T, C, 0, p(s["time_decay"]), p(s["time_first"]), p(s["k"]), p(s["v"]),
+                                 p(s_in), p(self.y), p(s_out), p(self.ckpt))
+        assert st == 0
+        st = self.L.wkv4_backward(self.stream, B, T, C, 0, p(s["time_decay"]), p(s["time_first"]), p(s["k"]), p(s["v"]),
+                                  p(s_in), p(s["dy"]), None, p(self.gtd), p(self.gtf), p(self.gk), p(self.gv),
+                                  p(self.gstate), p(self.ckpt), p(self.ws), self.ws.numel())
+        assert st == 0
+
+    def kernel_ids(self):
+        return {"forward": (3,), "backward": (4,)}
+
+
+def time_kernel(runner, kid, steps):
+    """Average launch duration (ms) of kernel `kid` over `steps` steps, by HIP
+    events recorded inside the library on the launch stream."""
+    L = runner.L
+    assert L.wkv_profile_begin(kid, steps) == 0
+    for _ in range(steps):
+        runner.step()
+    runner.torch.cuda.synchronize()
+    buf = (ctypes.c_float * steps)()
+    n = L.wkv_profile_end(buf, steps)
+    if n == 0:
+        return None
+    return sum(buf[:n]) / n
+
+
+def cpu_baseline(cfg, heads):
+    """The CPU restatement of the reference's pure-PyTorch path (chunk 128,
+    fp64 intra-chunk), fwd + autograd bwd, timed on the host cores on a head
+    subset of the same workload (heads are independent, cost is linear)."""
+    import torch
+    from oracle import wkv56 as O
+    from rwkv_wkv_hip import configs
+    spec = configs.SHAPES[cfg]
+    if spec["version"] == 4:
+        return None
+    ncores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    ncores = min(ncores, 16)
+    torch.set_num_threads(ncores)
+    B, T, H = spec["B"], spec["T"], spec["H"]
+    hs = min(heads, H)
+    bs = 1
+    wl = configs.make(cfg, B=bs, H=hs, C=hs * 64)
+    t = wl.tensors
+    v = spec["version"]
+    run = lambda: O.wkv_op_grads(v, bs, T, hs * 64, hs, t["r"].float(), t["k"].float(), t["v"].float(), t["w"], t["u"],
+                                 t["state"], t["dy"].float(), t["dstate"])
+    run()
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_all < 10 and len(times) < 8):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    tok_s = (bs * T) / (med * (H / hs))            # scaled to all heads of the layer; per batch row
+    out = {"value": tok_s, "unit": "tokens/s", "cores": ncores, "kind": "port",
+           "sample": (f"CPU restatement of rwkv_inner (chunk_len 128, fp64 intra-chunk, eager torch "
+                      f"{torch.__version__}) fwd + autograd bwd on {hs} of {H} heads of one batch row, T={T}; "
+                      f"median of {len(times)} runs = {med:.3f} s, scaled by {H}/{hs} heads"),
+           "threads": torch.get_num_threads()}
+    # the reference's own CPU-runnable case: WKV5 forward only, B1 T512 C768 H12 fp32
+    w0 = configs.make(0)
+    t0s = w0.tensors
+    f0 = lambda: O.wkv5_op(1, 512, 768, 12, t0s["state"], t0s["r"], t0s["k"], t0s["v"], t0s["w"], t0s["u"])
+    with torch.no_grad():
+        f0()
+        ts = []
+        for _ in range(5):
+            a = time.perf_counter()
+            f0()
+            ts.append(time.perf_counter() - a)
+    ts.sort()
+    out["cfg0_forward_tokens_per_s"] = 512 / ts[2]
+    return out
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU only (every (batch, head) recurrence is independent; "
+              "no multi-GPU path is part of it); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    runner = (Runner4 if a.cfg == 2 else Runner56)(a.cfg, a.algo, a.rotate)
+
+    for _ in range(a.warmup):
+        runner.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        runner.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt / a.steps * 1e3
+    tok_s = runner.tokens_per_step * a.steps / dt
+
+    # per-kernel launch durations (HIP events around the kernel, on its stream)
+    ksteps = min(a.steps, 20)
+    kern = {}
+    for phase, ids in runner.kernel_ids().items():
+        for kid in ids:
+            ms = time_kernel(runner, kid, ksteps)
+            if ms is not None:
+                kern[phase] = {"kernel_id": kid, "ms": ms}
+    dom = max(kern, key=lambda k: kern[k]["ms"])
+    dom_bytes = runner.bytes_bwd if dom == "backward" else runner.bytes_fwd
+    achieved = dom_bytes / (kern[dom]["ms"] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "kernel": f"{dom} (kernel id {kern[dom]['kernel_id']})",
+                "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_ms": kern[dom]["ms"],
+                "kernels_ms": {k: v["ms"] for k, v in kern.items()},
+                "whole_step_GBs": runner.bytes_step / (ms_step * 1e-3) / 1e9,
+                "whole_step_frac": runner.bytes_step / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    out = {"metric": "WKV fwd+bwd tokens/sec at v6-7B shape (1 GPU); % of peak HBM GB/s" if a.cfg == 4
+           else f"WKV fwd+bwd tokens/sec (cfg{a.cfg})",
+           "value": tok_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+           "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": runner.dtype_name, "data": "synthetic",
+           "config": {"workload": runner.desc, "algo": a.algo},
+           "roofline": roofline}
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(a.cfg, a.cpu_heads)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

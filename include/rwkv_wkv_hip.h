@@ -52,6 +52,22 @@ typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
 const char *wkv_strerror(int status);
 int wkv_abi_version(void);
 
+/* Timing hook for benchmarks (no counterpart in the reference).
+ * wkv_profile_begin: from now on the first `max_launches` launches of the
+ * kernel `kernel_id` are bracketed by HIP events recorded on the stream the
+ * kernel is launched on (the events are created here, not in the operators).
+ * wkv_profile_end: waits for those events, writes the elapsed milliseconds of
+ * each recorded launch to the HOST array ms[capacity], returns how many, and
+ * switches the hook off.  Not thread-safe; for single-threaded benchmark loops. */
+#define WKV_KERNEL_REC_FORWARD    1   /* per-token WKV5/6 forward  */
+#define WKV_KERNEL_REC_BACKWARD   2   /* per-token WKV5/6 backward */
+#define WKV_KERNEL_V4_FORWARD     3
+#define WKV_KERNEL_V4_BACKWARD    4
+#define WKV_KERNEL_CHUNK_FORWARD  10  /* chunked WKV5/6 forward    */
+#define WKV_KERNEL_CHUNK_BACKWARD 11  /* chunked WKV5/6 backward   */
+int wkv_profile_begin(int kernel_id, int max_launches);
+int wkv_profile_end(float *ms, int capacity);
+
 /* ---------------------------------------------------------------- WKV6 ----
  * Replaces wkv6state_cuda forward/backward as bound in
  * RWKV-v6/src/module/cuda/wkv6state_op.cpp:5-17 and called from

@@ -97,6 +97,35 @@ const char *wkv_strerror(int status) {
 
 int wkv_abi_version(void) { return 1; }
 
+int wkv_profile_begin(int kernel_id, int max_launches) {
+    ProfileSlot &p = profile_slot();
+    for (hipEvent_t e : p.start) (void)hipEventDestroy(e);
+    for (hipEvent_t e : p.stop) (void)hipEventDestroy(e);
+    p.start.clear(); p.stop.clear(); p.used = 0; p.id = KID_NONE;
+    if (kernel_id == KID_NONE || max_launches <= 0) return WKV_OK;
+    for (int i = 0; i < max_launches; i++) {
+        hipEvent_t a, b;
+        if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return WKV_ERR_LAUNCH;
+        p.start.push_back(a); p.stop.push_back(b);
+    }
+    p.id = kernel_id;
+    return WKV_OK;
+}
+
+int wkv_profile_end(float *ms, int capacity) {
+    ProfileSlot &p = profile_slot();
+    int n = 0;
+    for (size_t i = 0; i < p.used && (int)i < capacity; i++) {
+        if (hipEventSynchronize(p.stop[i]) != hipSuccess) break;
+        float t = 0.f;
+        if (hipEventElapsedTime(&t, p.start[i], p.stop[i]) != hipSuccess) break;
+        if (ms) ms[n] = t;
+        n++;
+    }
+    wkv_profile_begin(KID_NONE, 0);
+    return n;
+}
+
 size_t wkv6_forward_workspace(int, int, int, int, int, int) { return 0; }
 size_t wkv5_forward_workspace(int, int, int, int, int, int) { return 0; }
 

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <vector>
 
 namespace wkv {
 
@@ -63,6 +64,26 @@ __device__ __forceinline__ float log_decay(float x, bool floor_decay, bool *floo
     bool f = floor_decay && (l < LOG_W_FLOOR);
     if (floored) *floored = f;
     return f ? LOG_W_FLOOR : l;
+}
+
+// ---- optional timing of one kernel with caller-owned HIP events (wkv_profile_events)
+enum KernelId {
+    KID_NONE = 0, KID_REC_FORWARD = 1, KID_REC_BACKWARD = 2, KID_V4_FORWARD = 3, KID_V4_BACKWARD = 4,
+    KID_CHUNK_FORWARD = 10, KID_CHUNK_BACKWARD = 11
+};
+struct ProfileSlot {
+    int id = KID_NONE;
+    std::vector<hipEvent_t> start, stop;
+    size_t used = 0;
+};
+inline ProfileSlot &profile_slot() { static ProfileSlot p; return p; }
+inline void prof_begin(int id, hipStream_t s) {
+    ProfileSlot &p = profile_slot();
+    if (p.id == id && p.used < p.start.size()) (void)hipEventRecord(p.start[p.used], s);
+}
+inline void prof_end(int id, hipStream_t s) {
+    ProfileSlot &p = profile_slot();
+    if (p.id == id && p.used < p.start.size()) { (void)hipEventRecord(p.stop[p.used], s); p.used++; }
 }
 
 // sum per-batch partials: in (B, n) -> out (n); fixed order, so repeatable

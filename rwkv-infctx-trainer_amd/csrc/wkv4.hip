@@ -166,8 +166,10 @@ template <class T>
 static hipError_t fwd(hipStream_t s, int B, int Tlen, int C, const float *td, const float *tf, const void *k,
                       const void *v, const float *s_in, void *y, float *s_out, float *ckpt) {
     const int BC = B * C;
+    prof_begin(KID_V4_FORWARD, s);
     hipLaunchKernelGGL((v4_forward<T>), dim3((BC + 63) / 64), dim3(64), 0, s, BC, Tlen, C, td, tf, (const T *)k,
                        (const T *)v, s_in, (T *)y, s_out, ckpt);
+    prof_end(KID_V4_FORWARD, s);
     return hipGetLastError();
 }
 
@@ -182,8 +184,10 @@ static hipError_t bwd(hipStream_t s, int B, int Tlen, int C, const float *td, co
         if (e != hipSuccess) return e;
         ckpt = own_ckpt;
     }
+    prof_begin(KID_V4_BACKWARD, s);
     hipLaunchKernelGGL((v4_backward<T>), dim3((BC + 63) / 64), dim3(64), 0, s, BC, Tlen, C, td, tf, (const T *)k,
                        (const T *)v, (const T *)gy, gs_out, ckpt, gw_part, gu_part, (T *)gk, (T *)gv, gs_in);
+    prof_end(KID_V4_BACKWARD, s);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gw_part, gtd);

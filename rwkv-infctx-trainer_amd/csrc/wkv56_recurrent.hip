@@ -77,8 +77,8 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
     __syncthreads();
     for (int t0 = 0; t0 < Tlen; t0 += CH) {
         if (t0 + CH < Tlen) fetch(t0 + CH);
-#pragma unroll 2
-        for (int t = 0; t < CH; t++) {
+        const int nt = min(CH, Tlen - t0);      // the last block may be short
+        for (int t = 0; t < nt; t++) {
             const float vj = s_v[t][j];
             float acc = 0.f;
 #pragma unroll
@@ -192,8 +192,8 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
     __syncthreads();
     for (int t0 = 0; t0 < Tlen; t0 += CH) {
         if (t0 + CH < Tlen) fetch(t0 + CH, false);
-#pragma unroll 2
-        for (int t = 0; t < CH; t++) {
+        const int nt = min(CH, Tlen - t0);
+        for (int t = 0; t < nt; t++) {
             const float ki = s_k[t][own], wi = PER_TOKEN_W ? s_w[t][own] : w_own;
             const float uk = u_own * ki;
             float acc = 0.f;
@@ -252,8 +252,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
     __syncthreads();
     for (int t0 = last0; t0 >= 0; t0 -= CH) {
         if (t0 - CH >= 0) fetch(t0 - CH, true);
-#pragma unroll 2
-        for (int t = CH - 1; t >= 0; t--) {
+        for (int t = min(CH, Tlen - t0) - 1; t >= 0; t--) {
             // row-owned part (row i = own)
             const float ri = s_r[t][own], ki = s_k[t][own], wi = PER_TOKEN_W ? s_w[t][own] : w_own;
             float accG = 0.f, accP = 0.f;
@@ -331,12 +330,14 @@ static hipError_t launch_fwd(hipStream_t s, bool per_token, int B, int Tlen, int
                              const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
                              int floor_decay) {
     dim3 grid(B * H), block(NT);
+    prof_begin(KID_REC_FORWARD, s);
     if (per_token)
         hipLaunchKernelGGL((rec_forward<T, true>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k, (const T *)v,
                            w, u, s_in, (T *)y, s_out, floor_decay);
     else
         hipLaunchKernelGGL((rec_forward<T, false>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
                            (const T *)v, w, u, s_in, (T *)y, s_out, floor_decay);
+    prof_end(KID_REC_FORWARD, s);
     return hipGetLastError();
 }
 
@@ -350,6 +351,7 @@ static hipError_t launch_bwd(hipStream_t s, bool per_token, int B, int Tlen, int
     float *gu_part = qbuf + (size_t)B * Tlen * C;
     float *gw_part = gu_part + (size_t)B * C;
     dim3 grid(B * H), block(NT);
+    prof_begin(KID_REC_BACKWARD, s);
     if (per_token)
         hipLaunchKernelGGL((rec_backward<T, true>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
                            (const T *)v, w, u, s_in, (const T *)gy, gs_out, (T *)gr, (T *)gk, (T *)gv, gw, gw_part,
@@ -358,6 +360,7 @@ static hipError_t launch_bwd(hipStream_t s, bool per_token, int B, int Tlen, int
         hipLaunchKernelGGL((rec_backward<T, false>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
                            (const T *)v, w, u, s_in, (const T *)gy, gs_out, (T *)gr, (T *)gk, (T *)gv, nullptr, gw_part,
                            gu_part, gs_in, qbuf, floor_decay);
+    prof_end(KID_REC_BACKWARD, s);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gu_part, gu);

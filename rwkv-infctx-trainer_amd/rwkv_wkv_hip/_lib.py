@@ -23,6 +23,8 @@ _I = c_int
 SIGNATURES = {
     "wkv_strerror": (c_char_p, [_I]),
     "wkv_abi_version": (_I, []),
+    "wkv_profile_begin": (_I, [_I, _I]),
+    "wkv_profile_end": (_I, [_P, _I]),
     "wkv6_forward_workspace": (c_size_t, [_I] * 6),
     "wkv6_forward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 8 + [_P, c_size_t]),
     "wkv6_backward_workspace": (c_size_t, [_I] * 6),
@@ -52,6 +54,7 @@ def lib():
             raise WKVError(
                 f"{LIB_PATH} is missing: build the HIP library first "
                 "(make -C rwkv-infctx-trainer_amd/csrc).  There is no CPU fallback.")
+        import torch  # noqa: F401  (first, so that both share one HIP runtime)
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)
