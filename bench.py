@@ -92,6 +92,8 @@ class Runner56:
         st = self.fwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
                       p(s["u"]), p(s_in), p(self.y), p(s_out), p(self.ws), self.ws.numel())
         assert st == 0, self.L.wkv_strerror(st)
+        if self.L.wkv6_forward_workspace(B, T, C, H, self.dt, self.algo) > 0:
+            flags |= self._lib.CHECKPOINTS_VALID      # forward left its checkpoints in self.ws
         st = self.bwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
                       p(s["u"]), p(s_in), p(s["dy"]), p(s["dstate"]), p(self.gr), p(self.gk), p(self.gv), p(self.gw),
                       p(self.gu), p(self.gstate_in), p(self.ws), self.ws.numel())

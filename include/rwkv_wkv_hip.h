@@ -44,6 +44,10 @@ typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
                                  training path does (RWKV-v5/src/module/rwkv_inner.py:40,48);
                                  the gradient w.r.t. a floored w is zero */
 
+#define WKV_CHECKPOINTS_VALID 2u   /* backward only: the workspace passed is the one the matching
+                                      forward call (same arguments, same algo) was given, so the
+                                      state checkpoints it left there are used instead of rebuilt */
+
 /* algorithm selector */
 #define WKV_ALGO_AUTO      0  /* chunked where it applies, else recurrent */
 #define WKV_ALGO_RECURRENT 1  /* per-token fp32 recurrence, any T, any dtype */
@@ -75,6 +79,11 @@ int wkv_profile_end(float *ms, int capacity);
  * RWKV-v6/src/module/rwkv_inner.py:10-115 (state in, state out, fp32 state,
  * full state gradient).
  */
+/* Workspaces: forward needs none; if it is given one of at least
+ * wkv6_forward_workspace() bytes (the chunked algorithm only) it leaves state
+ * checkpoints there.  Passing that same buffer, sized by
+ * wkv6_backward_workspace() (>= the forward size), to backward together with
+ * WKV_CHECKPOINTS_VALID saves backward one sweep over k, v, w. */
 size_t wkv6_forward_workspace(int B, int T, int C, int H, int dtype, int algo);
 int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
                  const void *r, const void *k, const void *v, const float *w, const float *u,

@@ -4,6 +4,7 @@
 #include "../../include/rwkv_wkv_hip.h"
 #include "common.h"
 #include "wkv56_recurrent.hip"
+#include "wkv56_chunked.hip"
 #include "wkv4.hip"
 #include "cumsum_decay.hip"
 
@@ -21,9 +22,13 @@ int check_dims56(int B, int T, int C, int H, int dtype) {
     return WKV_OK;
 }
 
-int pick_algo56(int algo, int T, int dtype) {
-    if (algo == WKV_ALGO_AUTO) return WKV_ALGO_RECURRENT;
+// the blocked matrix-core path takes bf16 streams; everything else goes token by token
+int pick_algo56(int algo, int T, int dtype, bool backward) {
+    (void)backward; (void)T;
+    const bool can_chunk = dtype == WKV_BF16;
+    if (algo == WKV_ALGO_AUTO) return can_chunk ? WKV_ALGO_CHUNKED : WKV_ALGO_RECURRENT;
     if (algo == WKV_ALGO_RECURRENT) return algo;
+    if (algo == WKV_ALGO_CHUNKED) return can_chunk ? algo : WKV_ERR_ALGO;
     return WKV_ERR_ALGO;
 }
 
@@ -36,16 +41,33 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
     for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
                           (const void *)state_out})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
-    const int a = pick_algo56(algo, T, dtype);
+    const int a = pick_algo56(algo, T, dtype, false);
     if (a < 0) return a;
-    (void)workspace; (void)workspace_bytes;
+    if (a == WKV_ALGO_CHUNKED) {
+        // with a workspace the state at the start of every 64-token step is left there for backward
+        float *ckpt = nullptr;
+        if (workspace) {
+            if (!aligned16(workspace)) return WKV_ERR_ALIGN;
+            if (workspace_bytes < chunked::checkpoint_bytes(B, T, H)) return WKV_ERR_WORKSPACE;
+            ckpt = (float *)workspace;
+        }
+        hipError_t e = chunked::forward_launch((hipStream_t)stream, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
+                                               state_out, ckpt, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+        return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+    }
     hipError_t e = recurrent_forward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
                                      state_out, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
 
+size_t forward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
+    if (check_dims56(B, T, C, H, dtype)) return 0;
+    return pick_algo56(algo, T, dtype, false) == WKV_ALGO_CHUNKED ? chunked::checkpoint_bytes(B, T, H) : 0;
+}
+
 size_t backward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
     if (check_dims56(B, T, C, H, dtype)) return 0;
+    if (pick_algo56(algo, T, dtype, true) == WKV_ALGO_CHUNKED) return chunked::backward_workspace(B, T, C, H);
     return recurrent_backward_workspace(B, T, C);
 }
 
@@ -60,10 +82,16 @@ int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dty
                           (const void *)gstate_out, (const void *)gr, (const void *)gk, (const void *)gv,
                           (const void *)gw, (const void *)gu, (const void *)gstate_in, (const void *)workspace})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
-    const int a = pick_algo56(algo, T, dtype);
+    const int a = pick_algo56(algo, T, dtype, true);
     if (a < 0) return a;
     if (!workspace) return WKV_ERR_NULL;
     if (workspace_bytes < backward56_workspace(B, T, C, H, dtype, algo)) return WKV_ERR_WORKSPACE;
+    if (a == WKV_ALGO_CHUNKED) {
+        hipError_t e = chunked::backward_launch((hipStream_t)stream, per_token, B, T, C, H, r, k, v, w, u, state_in, gy,
+                                                gstate_out, gr, gk, gv, gw, gu, gstate_in, workspace,
+                                                (flags & WKV_CHECKPOINTS_VALID) != 0, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+        return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+    }
     hipError_t e = recurrent_backward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, gy,
                                       gstate_out, gr, gk, gv, gw, gu, gstate_in, (float *)workspace,
                                       (flags & WKV_FLOOR_DECAY) ? 1 : 0);
@@ -126,8 +154,12 @@ int wkv_profile_end(float *ms, int capacity) {
     return n;
 }
 
-size_t wkv6_forward_workspace(int, int, int, int, int, int) { return 0; }
-size_t wkv5_forward_workspace(int, int, int, int, int, int) { return 0; }
+size_t wkv6_forward_workspace(int B, int T, int C, int H, int dtype, int algo) {
+    return forward56_workspace(B, T, C, H, dtype, algo);
+}
+size_t wkv5_forward_workspace(int B, int T, int C, int H, int dtype, int algo) {
+    return forward56_workspace(B, T, C, H, dtype, algo);
+}
 
 int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
                  const void *k, const void *v, const float *w, const float *u, const float *state_in, void *y,

@@ -16,11 +16,13 @@ __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16 x) { return __uint_as_float((uint32_t)x.bits << 16); }
 __device__ __forceinline__ float to_float(f16 x) { return (float)x.h; }
 
-__device__ __forceinline__ uint16_t bf16_bits(float f) {     // round to nearest even
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;     // NaN
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+// fp32 -> bf16, round to nearest even (one v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint16_t bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+__device__ __forceinline__ uint32_t bf16_pack2(float lo, float hi) {      // lo in bits 0..15
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 h2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2));
 }
 
 template <class T> __device__ __forceinline__ T from_float(float f);
@@ -48,8 +50,8 @@ __device__ __forceinline__ void store4(float *p, const float (&o)[4]) {
 }
 __device__ __forceinline__ void store4(bf16 *p, const float (&o)[4]) {
     uint2 x;
-    x.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
-    x.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+    x.x = bf16_pack2(o[0], o[1]);
+    x.y = bf16_pack2(o[2], o[3]);
     *reinterpret_cast<uint2 *>(p) = x;
 }
 __device__ __forceinline__ void store4(f16 *p, const float (&o)[4]) {

@@ -1,0 +1,748 @@
+// WKV5 / WKV6 in blocked form on the matrix cores (bf16 operands, fp32 state).
+//
+// One workgroup of 4 wavefronts per (batch, head) walks the sequence in blocks
+// of 16 tokens.  Inside a block, with incl_t / excl_t the inclusive / exclusive
+// running sums of log w from the block's start, b their total and m = excl_8:
+//
+//   y_t = (r_t e^{excl_t}) S  +  sum_{s<t} [(r_t e^{excl_t-m}) . (k_s e^{m-incl_s})] v_s
+//         + (r_t . u k_t) v_t
+//   S  <- e^{b} o S + sum_s (k_s e^{b-incl_s})^T v_s
+//
+// Every exponent above is bounded (|.| <= 8 * 5.3 for the two re-centred
+// factors, <= 0 for the rest, because log w >= ln 0.005), so all factors fit
+// bf16/fp32 without the fp64 the reference needs for its 128-token chunks
+// (RWKV-v5/src/module/rwkv_inner.py:91-93).  The four contractions are
+// 16x16x16 bf16 MFMAs; the state lives in MFMA accumulators for the whole
+// sequence: wavefront w owns value columns 16w..16w+15 of S (all 64 key rows).
+//
+// The scaled operands are prepared 64 tokens at a time (lane = one channel of
+// one 16-token block: running sum in registers, no cross-lane scan) and laid
+// out in LDS so that every MFMA operand fragment is one 8-byte read; rows are
+// padded to 68 elements, which spreads the 16 rows of a fragment over all banks.
+#include "common.h"
+
+namespace wkv {
+namespace chunked {
+
+typedef short s4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int SB = 64;        // tokens prepared per staging step
+constexpr int LD = 68;        // padded row length of a 64x64 bf16 tile in LDS
+constexpr int NT = 256;
+
+typedef short s8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+
+// D[m][n] += sum_k A[m][k] B[k][n] for one 16-deep product.  Issued as a 16x16x32 MFMA
+// with a zero upper half: on gfx950 a 16x16x16 MFMA chained on the accumulator of a
+// 16x16x32 one returned corrupted rows in this kernel, and both cost one issue slot.
+__device__ __forceinline__ f4 mma(s4 a, s4 b, f4 c) {
+    const s8 av = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
+    const s8 bv = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, av), __builtin_bit_cast(b8, bv), c, 0, 0, 0);
+}
+// two 16-deep products in one 16x16x32 instruction: D += A0 B0 + A1 B1
+__device__ __forceinline__ f4 mma2(s4 a0, s4 a1, s4 b0, s4 b1, f4 c) {
+    const s8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+    const s8 b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
+}
+// lane (g = lane/16, n = lane%16) supplies A[n][4g..4g+3] and B[4g..4g+3][n], receives D[4g..4g+3][n]
+__device__ __forceinline__ s4 frag(const uint16_t *tile, int row, int col) {
+    return *reinterpret_cast<const s4 *>(tile + row * LD + col);
+}
+__device__ __forceinline__ float bf2f(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ float bf_lo(uint32_t p) { return __uint_as_float(p << 16); }          // element 0 of a pair
+__device__ __forceinline__ float bf_hi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }  // element 1
+__device__ __forceinline__ s4 as_s4(uint32_t a, uint32_t b) {
+    const uint2 x = make_uint2(a, b);
+    return __builtin_bit_cast(s4, x);
+}
+__device__ __forceinline__ s4 pack(f4 x) { return as_s4(bf16_pack2(x[0], x[1]), bf16_pack2(x[2], x[3])); }
+// x ~= hi + lo with both parts bf16: 16 mantissa bits instead of 8
+__device__ __forceinline__ void split2(float a, float b, uint32_t &hi, uint32_t &lo) {
+    hi = bf16_pack2(a, b);
+    lo = bf16_pack2(a - bf_lo(hi), b - bf_hi(hi));
+}
+__device__ __forceinline__ void split4(f4 x, s4 &hi, s4 &lo) {
+    uint32_t h0, l0, h1, l1;
+    split2(x[0], x[1], h0, l0);
+    split2(x[2], x[3], h1, l1);
+    hi = as_s4(h0, h1);
+    lo = as_s4(l0, l1);
+}
+
+// sum each of 8 per-lane values over the 32 lanes of a half wavefront; afterwards
+// lane L holds the total of value index 4*b4 + 2*b3 + b2 (bK = bit K of L)
+__device__ __forceinline__ float sum8_over_half(const float (&p)[8], int lane) {
+    float a4[4], a2[2];
+    const bool h4 = lane & 16, h3 = lane & 8, h2 = lane & 4;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const float keep = h4 ? p[e + 4] : p[e], send = h4 ? p[e] : p[e + 4];
+        a4[e] = keep + __shfl_xor(send, 16);
+    }
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        const float keep = h3 ? a4[e + 2] : a4[e], send = h3 ? a4[e] : a4[e + 2];
+        a2[e] = keep + __shfl_xor(send, 8);
+    }
+    const float keep = h2 ? a2[1] : a2[0], send = h2 ? a2[0] : a2[1];
+    float x = keep + __shfl_xor(send, 4);
+    x += __shfl_xor(x, 2);
+    x += __shfl_xor(x, 1);
+    return x;
+}
+__device__ __forceinline__ int sum8_index(int lane) { return ((lane >> 4) & 1) * 4 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1); }
+
+// collects 8 tokens of a channel pair (one packed pair per token) into two rows of a [channel][token] tile
+struct Gather8 {
+    uint32_t a[4], b[4];
+    __device__ __forceinline__ void add(int x, uint32_t pair) {
+        if (x & 1) { a[x >> 1] |= pair << 16;   b[x >> 1] |= pair & 0xffff0000u; }
+        else       { a[x >> 1] = pair & 0xffffu; b[x >> 1] = pair >> 16; }
+    }
+    __device__ __forceinline__ void put(uint16_t *tile, int ot) const {
+        *reinterpret_cast<uint2 *>(&tile[ot]) = make_uint2(a[0], a[1]);
+        *reinterpret_cast<uint2 *>(&tile[ot + 4]) = make_uint2(a[2], a[3]);
+        *reinterpret_cast<uint2 *>(&tile[ot + LD]) = make_uint2(b[0], b[1]);
+        *reinterpret_cast<uint2 *>(&tile[ot + LD + 4]) = make_uint2(b[2], b[3]);
+    }
+};
+
+struct FwdTiles {
+    uint16_t rd[SB * LD];    // r e^{excl-m}     [token][channel]  (bf16 head of the value)
+    uint16_t rdl[SB * LD];   //                                    (bf16 remainder)
+    uint16_t kd[SB * LD];    // k e^{m-incl}     [token][channel]
+    uint16_t kdl[SB * LD];
+    uint16_t rh[SB * LD];    // r e^{excl}       [token][channel]
+    uint16_t rhl[SB * LD];
+    uint16_t khT[SB * LD];   // k e^{b-incl}     [channel][token]
+    uint16_t khTl[SB * LD];
+    uint16_t vT[SB * LD];    // v                [channel][token]
+    float dec[4][HEAD];      // e^{b} per block and channel
+    float rho[SB];           // r . (u o k) per token
+};
+
+// Forward over tokens [0, Tlen) of one (batch, head).  ckpt (optional) receives
+// the state at the start of every 64-token step, [bh][step][key][value] fp32.
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
+        const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
+        const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
+        bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, int floor_decay)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    FwdTiles &sm = *reinterpret_cast<FwdTiles *>(smem_raw);
+    const int bh = blockIdx.x, b = bh / H, h = bh % H;
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    const int nsb = (Tlen + SB - 1) / SB;
+
+    // state tiles: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]
+    f4 S[4];
+    {
+        const float *sp = s_in + (size_t)bh * HEAD * HEAD;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
+    }
+    // staging role: block wv of the step, tokens 8*half..8*half+7 of it, channels c0, c0+1
+    const int half = lane >> 5, c0 = 2 * (lane & 31);
+    const float2 u_c = *reinterpret_cast<const float2 *>(u + h * HEAD + c0);
+    float2 l_const = make_float2(0.f, 0.f);
+    if (!PER_TOKEN_W) {
+        l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
+        l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
+    }
+
+    uint32_t pr[8], pk[8], pv[8];
+    float2 pw[8];
+    auto fetch = [&](int sb) {
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+            const int t = sb * SB + 16 * wv + 8 * half + x;
+            if (t < Tlen) {
+                const size_t o = base + (size_t)t * C + c0;
+                pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
+                pk[x] = *reinterpret_cast<const uint32_t *>(k + o);
+                pv[x] = *reinterpret_cast<const uint32_t *>(v + o);
+                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
+            } else {
+                pr[x] = pk[x] = pv[x] = 0;
+                pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);   // log w = 0
+            }
+        }
+    };
+
+    fetch(0);
+    for (int sb = 0; sb < nsb; sb++) {
+        // ---------------- prepare the scaled operands of 64 tokens
+        {
+            float ia[8], ib[8], la[8], lb[8];
+            float ra = 0.f, rb = 0.f;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                la[x] = PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
+                lb[x] = PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
+                ra += la[x]; rb += lb[x];
+                ia[x] = ra; ib[x] = rb;
+            }
+            // the other half of the block sits in lane ^ 32
+            const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
+            const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
+            const float tota = ra + oa, totb = rb + ob;
+            const float mida = half ? oa : ra, midb = half ? ob : rb;       // running sum after 8 tokens
+            const float ea_nm = __expf(-mida), eb_nm = __expf(-midb);
+            const float ea_mb = __expf(mida - tota), eb_mb = __expf(midb - totb);
+            float p[8];
+            Gather8 gk_h, gk_l, gv_;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                const float inca = ia[x] + offa, incb = ib[x] + offb;
+                const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]), kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
+                const float rha = rfa * __expf(inca - la[x]), rhb = rfb * __expf(incb - lb[x]);
+                const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
+                const int o = (16 * wv + 8 * half + x) * LD + c0;
+                uint32_t hi, lo;
+                split2(rha, rhb, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
+                split2(rha * ea_nm, rhb * eb_nm, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.rd[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.rdl[o]) = lo;
+                split2(kha * ea_mb, khb * eb_mb, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.kd[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.kdl[o]) = lo;
+                p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
+                split2(kha, khb, hi, lo);
+                gk_h.add(x, hi);
+                gk_l.add(x, lo);
+                gv_.add(x, pv[x]);
+            }
+            const int ot = c0 * LD + 16 * wv + 8 * half;
+            gk_h.put(sm.khT, ot);
+            gk_l.put(sm.khTl, ot);
+            gv_.put(sm.vT, ot);
+            if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(tota), __expf(totb));
+            const float tot_p = sum8_over_half(p, lane);
+            if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
+        }
+        __syncthreads();
+        if (sb + 1 < nsb) fetch(sb + 1);          // next step's loads fly during the MFMA phase
+
+        // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
+        if (ckpt) {
+            float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) cp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (sb * SB + 16 * q >= Tlen) break;
+            // A^T[s][t] = sum_i kd[s][i] rd[t][i]; lane gets s = 4g+e, t = n
+            // (operands carried as bf16 head + remainder; head*head + rem*head + head*rem)
+            f4 at = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                const int row = 16 * q + n, c0 = 16 * kk + 4 * g, c1 = c0 + 16;
+                const s4 kh0 = frag(sm.kd, row, c0), kh1 = frag(sm.kd, row, c1);
+                const s4 rh0 = frag(sm.rd, row, c0), rh1 = frag(sm.rd, row, c1);
+                at = mma2(kh0, kh1, rh0, rh1, at);
+                at = mma2(frag(sm.kdl, row, c0), frag(sm.kdl, row, c1), rh0, rh1, at);
+                at = mma2(kh0, kh1, frag(sm.rdl, row, c0), frag(sm.rdl, row, c1), at);
+            }
+            const float rho_t = sm.rho[16 * q + n];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int s = 4 * g + e;
+                at[e] = s < n ? at[e] : (s == n ? rho_t : 0.f);
+            }
+            s4 a_hi, a_lo;                                  // A[t = n][s = 4g..4g+3]
+            split4(at, a_hi, a_lo);
+            const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
+            f4 yt = {0.f, 0.f, 0.f, 0.f};
+            yt = mma2(a_hi, a_lo, v_op, v_op, yt);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                s4 s0h, s0l, s1h, s1l;
+                split4(S[kk], s0h, s0l);
+                split4(S[kk + 1], s1h, s1l);
+                const int row = 16 * q + n, ca = 16 * kk + 4 * g, cb = ca + 16;
+                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                yt = mma2(r0, r1, s0h, s1h, yt);
+                yt = mma2(r0, r1, s0l, s1l, yt);
+                yt = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, yt);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int t = sb * SB + 16 * q + 4 * g + e;
+                if (y && t < Tlen) y[base + (size_t)t * C + 16 * wv + n] = bf16{bf16_bits(yt[e])};
+            }
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
+                S[kk][0] *= d4.x; S[kk][1] *= d4.y; S[kk][2] *= d4.z; S[kk][3] *= d4.w;
+                S[kk] = mma2(frag(sm.khT, 16 * kk + n, 16 * q + 4 * g), frag(sm.khTl, 16 * kk + n, 16 * q + 4 * g),
+                             v_op, v_op, S[kk]);
+            }
+        }
+        __syncthreads();
+    }
+    if (s_out) {
+        float *op = s_out + (size_t)bh * HEAD * HEAD;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) op[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+    }
+}
+
+
+// ------------------------------------------------------------------ backward --
+// Walks the 64-token steps from the last to the first.  Per step: prepare the
+// operands, rebuild the state at the start of each of its four blocks from the
+// step's checkpoint, then take the blocks in reverse.  With G the gradient of
+// the state at a block's end, P[t][s] = gy_t . v_s, rh = r e^{excl}, kh = k e^{b-incl}:
+//
+//   gr_t = e^{excl_t} (gy_t S^T) + e^{excl_t-b} sum_{s<t} P[t][s] kh_s + u k_t P[t][t]
+//   gk_s = e^{-incl_s} sum_{t>s} P[t][s] rh_t + e^{b-incl_s} (v_s G^T) + u r_s P[s][s]
+//   gv_s = sum_{t>=s} A~[t][s] gy_t + kh_s G          (A~ = the forward's masked matrix)
+//   G   <- e^{b} o G + rh^T gy
+//
+// and the decay gradient from the running sum  A_{t-1} = A_t + r_t gr_t - k_t gk_t,
+// dL/dlog w_t = A_t - k_t (gk_t - u r_t P[t][t]),  re-anchored at every step end
+// to sum_j G o S.  Each wavefront owns key channels 16w..16w+15 for gr, gk, gw
+// (state and G held value-major for that slice) and value channels 16w..16w+15
+// for gv (a second copy of G, key-major), so no result crosses wavefronts.
+struct BwdTiles {
+    uint16_t gy[SB * LD];    // gy              [token][value]
+    uint16_t v[SB * LD];     // v               [token][value]
+    uint16_t rd[SB * LD];    // r e^{excl-m}    [token][key]   head / remainder
+    uint16_t rdl[SB * LD];
+    uint16_t kd[SB * LD];    // k e^{m-incl}    [token][key]
+    uint16_t kdl[SB * LD];
+    uint16_t kh[SB * LD];    // k e^{b-incl}    [token][key]
+    uint16_t khl[SB * LD];
+    uint16_t gyT[SB * LD];   // gy              [value][token]
+    uint16_t vT[SB * LD];    // v               [value][token]
+    uint16_t khT[SB * LD];   // k e^{b-incl}    [key][token]
+    uint16_t khTl[SB * LD];
+    uint16_t rhT[SB * LD];   // r e^{excl}      [key][token]
+    uint16_t rhTl[SB * LD];
+    float incl[SB * HEAD];   // inclusive running log decay inside the block [token][key]
+    float lw[SB * HEAD];     // log w                                         [token][key]
+    float tot[4][HEAD];      // b per block and key
+    float dec[4][HEAD];      // e^{b}
+    float rho[SB];
+};
+
+__device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane groups of 16
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
+}
+
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
+        const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
+        const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
+        const float *__restrict__ gs_out, const float *__restrict__ ckpt,
+        bf16 *__restrict__ gr, bf16 *__restrict__ gk, bf16 *__restrict__ gv, float *__restrict__ gw_tok,
+        float *__restrict__ gw_part, float *__restrict__ gu_part, float *__restrict__ gs_in, int floor_decay)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    BwdTiles &sm = *reinterpret_cast<BwdTiles *>(smem_raw);
+    const int bh = blockIdx.x, b = bh / H, h = bh % H;
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    const int nsb = (Tlen + SB - 1) / SB;
+    const int own = 16 * wv + n;                 // key channel (gr, gk, gw) / value channel (gv) of this lane
+    const float u_i = u[h * HEAD + own];
+
+    // GT[kk][e] = G[key own][value 16kk+4g+e];  GJ[kk][e] = G[key 16kk+4g+e][value own]
+    f4 GT[4], GJ[4];
+    {
+        const float *gp = gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                GT[kk][e] = gp ? gp[own * HEAD + 16 * kk + 4 * g + e] : 0.f;
+                GJ[kk][e] = gp ? gp[(16 * kk + 4 * g + e) * HEAD + own] : 0.f;
+            }
+    }
+    float A_run = 0.f, gu_acc = 0.f, gw_acc = 0.f;
+
+    // staging role (as in forward): block wv, tokens 8*half.., channels c0, c0+1
+    const int half = lane >> 5, c0 = 2 * (lane & 31);
+    const float2 u_c = *reinterpret_cast<const float2 *>(u + h * HEAD + c0);
+    float2 l_const = make_float2(0.f, 0.f);
+    if (!PER_TOKEN_W) {
+        l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
+        l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
+    }
+    uint32_t pr[8], pk[8], pv[8], pg[8];
+    float2 pw[8];
+    auto fetch = [&](int sb) {
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+            const int t = sb * SB + 16 * wv + 8 * half + x;
+            if (t < Tlen) {
+                const size_t o = base + (size_t)t * C + c0;
+                pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
+                pk[x] = *reinterpret_cast<const uint32_t *>(k + o);
+                pv[x] = *reinterpret_cast<const uint32_t *>(v + o);
+                pg[x] = *reinterpret_cast<const uint32_t *>(gy + o);
+                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
+            } else {
+                pr[x] = pk[x] = pv[x] = pg[x] = 0;
+                pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);
+            }
+        }
+    };
+
+    fetch(nsb - 1);
+    for (int sb = nsb - 1; sb >= 0; sb--) {
+        // ---------------- prepare the operands of 64 tokens
+        {
+            float ia[8], ib[8], la[8], lb[8];
+            float ra = 0.f, rb = 0.f;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                la[x] = PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
+                lb[x] = PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
+                ra += la[x]; rb += lb[x];
+                ia[x] = ra; ib[x] = rb;
+            }
+            const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
+            const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
+            const float tota = ra + oa, totb = rb + ob;
+            const float mida = half ? oa : ra, midb = half ? ob : rb;
+            const float ea_nm = __expf(-mida), eb_nm = __expf(-midb);
+            const float ea_mb = __expf(mida - tota), eb_mb = __expf(midb - totb);
+            float p[8];
+            Gather8 gk_h, gk_l, gr_h, gr_l, gv_, gg_;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                const float inca = ia[x] + offa, incb = ib[x] + offb;
+                const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]), kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
+                const float rha = rfa * __expf(inca - la[x]), rhb = rfb * __expf(incb - lb[x]);
+                const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
+                const int tk = 16 * wv + 8 * half + x;
+                const int o = tk * LD + c0;
+                uint32_t hi, lo;
+                *reinterpret_cast<uint32_t *>(&sm.gy[o]) = pg[x];
+                *reinterpret_cast<uint32_t *>(&sm.v[o]) = pv[x];
+                split2(rha * ea_nm, rhb * eb_nm, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.rd[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.rdl[o]) = lo;
+                split2(kha * ea_mb, khb * eb_mb, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.kd[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.kdl[o]) = lo;
+                split2(kha, khb, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.kh[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.khl[o]) = lo;
+                gk_h.add(x, hi);
+                gk_l.add(x, lo);
+                split2(rha, rhb, hi, lo);
+                gr_h.add(x, hi);
+                gr_l.add(x, lo);
+                gv_.add(x, pv[x]);
+                gg_.add(x, pg[x]);
+                *reinterpret_cast<float2 *>(&sm.incl[tk * HEAD + c0]) = make_float2(inca, incb);
+                *reinterpret_cast<float2 *>(&sm.lw[tk * HEAD + c0]) = make_float2(la[x], lb[x]);
+                p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
+            }
+            const int ot = c0 * LD + 16 * wv + 8 * half;
+            gk_h.put(sm.khT, ot);
+            gk_l.put(sm.khTl, ot);
+            gr_h.put(sm.rhT, ot);
+            gr_l.put(sm.rhTl, ot);
+            gv_.put(sm.vT, ot);
+            gg_.put(sm.gyT, ot);
+            if (!half) {
+                *reinterpret_cast<float2 *>(&sm.tot[wv][c0]) = make_float2(tota, totb);
+                *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(tota), __expf(totb));
+            }
+            const float tot_p = sum8_over_half(p, lane);
+            if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
+        }
+        __syncthreads();
+        if (sb > 0) fetch(sb - 1);
+
+        // ---------------- rebuild the state at the start of each block (value-major slice: key `own`)
+        f4 ST[4];
+        {
+            const float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD + own * HEAD;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const float4 x = *reinterpret_cast<const float4 *>(cp + 16 * kk + 4 * g);
+                ST[kk][0] = x.x; ST[kk][1] = x.y; ST[kk][2] = x.z; ST[kk][3] = x.w;
+            }
+        }
+        s4 Sh[4][4], Sl[4][4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) split4(ST[kk], Sh[q][kk], Sl[q][kk]);
+            if (sb * SB + 16 * q >= Tlen) continue;
+            const float dq = sm.dec[q][own];
+            const s4 khf = frag(sm.khT, own, 16 * q + 4 * g), khfl = frag(sm.khTl, own, 16 * q + 4 * g);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                ST[kk] = ST[kk] * dq;
+                const s4 vf_ = frag(sm.vT, 16 * kk + n, 16 * q + 4 * g);
+                ST[kk] = mma2(vf_, vf_, khf, khfl, ST[kk]);
+            }
+        }
+        {   // anchor of the decay-gradient sum at the end of this step: sum_j G o S
+            float a = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) a = fmaf(GT[kk][e], ST[kk][e], a);
+            A_run = group_sum4(a);
+        }
+
+        // ---------------- the four blocks, last first
+#pragma unroll
+        for (int q = 3; q >= 0; q--) {
+            if (sb * SB + 16 * q >= Tlen) continue;
+            const int row = 16 * q + n;
+            s4 gyf[4], vf[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                gyf[kk] = frag(sm.gy, row, 16 * kk + 4 * g);
+                vf[kk] = frag(sm.v, row, 16 * kk + 4 * g);
+            }
+            // pt[e] = P[t = 4g+e][s = n],  ptT[e] = P[t = n][s = 4g+e]
+            f4 pt = {0.f, 0.f, 0.f, 0.f}, ptT = {0.f, 0.f, 0.f, 0.f};
+            pt = mma2(gyf[0], gyf[1], vf[0], vf[1], pt);
+            pt = mma2(gyf[2], gyf[3], vf[2], vf[3], pt);
+            ptT = mma2(vf[0], vf[1], gyf[0], gyf[1], ptT);
+            ptT = mma2(vf[2], vf[3], gyf[2], gyf[3], ptT);
+            float pd[4];                                   // P[t][t] for this lane's tokens t = 4g+e
+            f4 pm, pTm;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                pd[e] = __shfl(pt[e], (lane & 48) | (4 * g + e));
+                pm[e] = (4 * g + e > n) ? pt[e] : 0.f;     // later tokens t > s
+                pTm[e] = (4 * g + e < n) ? ptT[e] : 0.f;   // earlier tokens s < t
+            }
+            s4 pm_h, pm_l, pT_h, pT_l;
+            split4(pm, pm_h, pm_l);
+            split4(pTm, pT_h, pT_l);
+
+            // the forward's masked matrix: at[e] = A~[t = 4g+e][s = n]
+            f4 at = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                const s4 rh0 = frag(sm.rd, row, ca), rh1 = frag(sm.rd, row, cb);
+                const s4 kh0 = frag(sm.kd, row, ca), kh1 = frag(sm.kd, row, cb);
+                at = mma2(rh0, rh1, kh0, kh1, at);
+                at = mma2(frag(sm.rdl, row, ca), frag(sm.rdl, row, cb), kh0, kh1, at);
+                at = mma2(rh0, rh1, frag(sm.kdl, row, ca), frag(sm.kdl, row, cb), at);
+            }
+            {
+                const float rho_s = sm.rho[16 * q + n];
+#pragma unroll
+                for (int e = 0; e < 4; e++) at[e] = (4 * g + e > n) ? at[e] : ((4 * g + e == n) ? rho_s : 0.f);
+            }
+            s4 a_h, a_l;
+            split4(at, a_h, a_l);
+
+            const s4 gyTf = frag(sm.gyT, own, 16 * q + 4 * g);     // gy[t = 4g..][value own]
+            const s4 khTf = frag(sm.khT, own, 16 * q + 4 * g);     // kh[s = 4g..][key own]
+            const s4 khTfl = frag(sm.khTl, own, 16 * q + 4 * g);
+            const s4 rhTf = frag(sm.rhT, own, 16 * q + 4 * g);     // rh[t = 4g..][key own]
+            const s4 rhTfl = frag(sm.rhTl, own, 16 * q + 4 * g);
+
+            // gv[s = 4g+e][value own]
+            f4 gvt = {0.f, 0.f, 0.f, 0.f};
+            gvt = mma2(a_h, a_l, gyTf, gyTf, gvt);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                s4 g0h, g0l, g1h, g1l;
+                split4(GJ[kk], g0h, g0l);
+                split4(GJ[kk + 1], g1h, g1l);
+                const s4 k0 = frag(sm.kh, row, 16 * kk + 4 * g), k1 = frag(sm.kh, row, 16 * kk + 16 + 4 * g);
+                gvt = mma2(k0, k1, g0h, g1h, gvt);
+                gvt = mma2(k0, k1, g0l, g1l, gvt);
+                gvt = mma2(frag(sm.khl, row, 16 * kk + 4 * g), frag(sm.khl, row, 16 * kk + 16 + 4 * g), g0h, g1h, gvt);
+            }
+            // gr, gk pieces at [token 4g+e][key own]
+            f4 q1 = {0.f, 0.f, 0.f, 0.f}, q2 = {0.f, 0.f, 0.f, 0.f}, q3 = {0.f, 0.f, 0.f, 0.f}, q4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                q1 = mma2(gyf[kk], gyf[kk + 1], Sh[q][kk], Sh[q][kk + 1], q1);
+                q1 = mma2(gyf[kk], gyf[kk + 1], Sl[q][kk], Sl[q][kk + 1], q1);
+                s4 g0h, g0l, g1h, g1l;
+                split4(GT[kk], g0h, g0l);
+                split4(GT[kk + 1], g1h, g1l);
+                q4 = mma2(vf[kk], vf[kk + 1], g0h, g1h, q4);
+                q4 = mma2(vf[kk], vf[kk + 1], g0l, g1l, q4);
+            }
+            q2 = mma2(pT_h, pT_l, khTf, khTf, q2);
+            q2 = mma(pT_h, khTfl, q2);
+            q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);
+            q3 = mma(pm_h, rhTfl, q3);
+
+            const float tot_i = sm.tot[q][own], mid_i = sm.incl[(16 * q + 7) * HEAD + own];
+            float c[4], z[4], lfac[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int tk = 16 * q + 4 * g + e;
+                const int t = sb * SB + tk;
+                const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
+                // r, k back from their re-centred head + remainder (16 mantissa bits)
+                const float rr = (bf2f(sm.rd[tk * LD + own]) + bf2f(sm.rdl[tk * LD + own])) * __expf(mid_i - exc);
+                const float kr = (bf2f(sm.kd[tk * LD + own]) + bf2f(sm.kdl[tk * LD + own])) * __expf(inc - mid_i);
+                const float grv = __expf(exc) * q1[e] + __expf(exc - tot_i) * q2[e] + u_i * kr * pd[e];
+                const float gkn = __expf(-inc) * q3[e] + __expf(tot_i - inc) * q4[e];
+                const float gkv = gkn + u_i * rr * pd[e];
+                c[e] = rr * grv - kr * gkv;
+                z[e] = kr * gkn;
+                lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
+                gu_acc = fmaf(rr * kr, pd[e], gu_acc);
+                if (t < Tlen) {
+                    const size_t o = base + (size_t)t * C;
+                    gr[o + own] = bf16{bf16_bits(grv)};
+                    gk[o + own] = bf16{bf16_bits(gkv)};
+                    gv[o + own] = bf16{bf16_bits(gvt[e])};
+                }
+            }
+            {   // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over later tokens of c
+                const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
+                const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
+                const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
+                const float all = group_sum4(mine);
+                const float suf[4] = {suf0, suf1, suf2, 0.f};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float Dt = A_run + later + suf[e] - z[e];
+                    const int t = sb * SB + 16 * q + 4 * g + e;
+                    if (PER_TOKEN_W) {
+                        if (t < Tlen) gw_tok[base + (size_t)t * C + own] = Dt * lfac[e];
+                    } else {
+                        gw_acc += (t < Tlen) ? Dt : 0.f;
+                    }
+                }
+                A_run += all;
+            }
+            // G <- e^{b} o G + rh^T gy, both copies
+            {
+                const float dq = sm.dec[q][own];
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    GT[kk] = GT[kk] * dq;
+                    const s4 gT_ = frag(sm.gyT, 16 * kk + n, 16 * q + 4 * g);
+                    GT[kk] = mma2(gT_, gT_, rhTf, rhTfl, GT[kk]);
+                    const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
+                    GJ[kk][0] *= d4.x; GJ[kk][1] *= d4.y; GJ[kk][2] *= d4.z; GJ[kk][3] *= d4.w;
+                    GJ[kk] = mma2(frag(sm.rhT, 16 * kk + n, 16 * q + 4 * g), frag(sm.rhTl, 16 * kk + n, 16 * q + 4 * g),
+                                  gyTf, gyTf, GJ[kk]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    if (gs_in) {
+        float *gp = gs_in + (size_t)bh * HEAD * HEAD + own * HEAD;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+            *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(GT[kk][0], GT[kk][1], GT[kk][2], GT[kk][3]);
+    }
+    gu_acc = group_sum4(gu_acc);
+    gw_acc = group_sum4(gw_acc);
+    if (g == 0) {
+        gu_part[(size_t)bh * HEAD + own] = gu_acc;
+        if (!PER_TOKEN_W) {
+            bool fl;
+            const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
+            gw_part[(size_t)bh * HEAD + own] = fl ? 0.f : gw_acc * l;
+        }
+    }
+}
+
+size_t checkpoint_bytes(int B, int Tlen, int H) {
+    return (size_t)B * H * ((Tlen + SB - 1) / SB) * HEAD * HEAD * sizeof(float);
+}
+
+hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
+                          const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
+                          float *ckpt, int floor_decay) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *)forward<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)sizeof(FwdTiles));
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void *)forward<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)sizeof(FwdTiles));
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    dim3 grid(B * H), block(NT);
+    prof_begin(KID_CHUNK_FORWARD, s);
+    if (per_token)
+        hipLaunchKernelGGL((forward<true>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, (const bf16 *)r, (const bf16 *)k,
+                           (const bf16 *)v, w, u, s_in, (bf16 *)y, s_out, ckpt, floor_decay);
+    else
+        hipLaunchKernelGGL((forward<false>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, (const bf16 *)r, (const bf16 *)k,
+                           (const bf16 *)v, w, u, s_in, (bf16 *)y, s_out, ckpt, floor_decay);
+    prof_end(KID_CHUNK_FORWARD, s);
+    return hipGetLastError();
+}
+
+// workspace of the backward call: checkpoints | gu partials (B,C) | gw partials (B,C)
+size_t backward_workspace(int B, int Tlen, int C, int H) {
+    return checkpoint_bytes(B, Tlen, H) + 2 * (size_t)B * C * sizeof(float);
+}
+
+hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
+                           const void *v, const float *w, const float *u, const float *s_in, const void *gy,
+                           const float *gs_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gs_in,
+                           void *workspace, bool have_ckpt, int floor_decay) {
+    float *ckpt = (float *)workspace;
+    float *gu_part = (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H));
+    float *gw_part = gu_part + (size_t)B * C;
+    if (!have_ckpt) {      // the forward call did not leave its checkpoints here: rebuild them
+        hipError_t e = forward_launch(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, ckpt, floor_decay);
+        if (e != hipSuccess) return e;
+    }
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *)backward<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)sizeof(BwdTiles));
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void *)backward<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)sizeof(BwdTiles));
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    dim3 grid(B * H), block(NT);
+    prof_begin(KID_CHUNK_BACKWARD, s);
+    if (per_token)
+        hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, (const bf16 *)r,
+                           (const bf16 *)k, (const bf16 *)v, w, u, (const bf16 *)gy, gs_out, ckpt, (bf16 *)gr,
+                           (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in, floor_decay);
+    else
+        hipLaunchKernelGGL((backward<false>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, (const bf16 *)r,
+                           (const bf16 *)k, (const bf16 *)v, w, u, (const bf16 *)gy, gs_out, ckpt, (bf16 *)gr,
+                           (bf16 *)gk, (bf16 *)gv, nullptr, gw_part, gu_part, gs_in, floor_decay);
+    prof_end(KID_CHUNK_BACKWARD, s);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gu_part, gu);
+    if (!per_token) hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gw_part, gw);
+    return hipGetLastError();
+}
+
+}  // namespace chunked
+}  // namespace wkv

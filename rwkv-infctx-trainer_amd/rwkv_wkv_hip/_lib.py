@@ -10,10 +10,11 @@ import os
 from ctypes import c_char_p, c_int, c_size_t, c_uint, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "librwkv_wkv_hip.so")
+LIB_PATH = os.environ.get("RWKV_WKV_LIB", os.path.join(_HERE, "librwkv_wkv_hip.so"))
 
 WKV_F32, WKV_BF16, WKV_F16 = 0, 1, 2
 FLOOR_DECAY = 1
+CHECKPOINTS_VALID = 2
 ALGO_AUTO, ALGO_RECURRENT, ALGO_CHUNKED = 0, 1, 2
 
 _P = c_void_p

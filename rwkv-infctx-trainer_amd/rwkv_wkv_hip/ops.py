@@ -64,22 +64,28 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
 
-def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32):
+def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad):
+    """Returns y, new_state and, when a backward call will follow, the
+    workspace in which the forward kernel left its state checkpoints (sized
+    for that backward call) together with the algorithm that was in force."""
     L = _lib.lib()
     dt = _check_rkv(B, T, C, H, r, k, v)
     _on_gpu(r, k, v, w32, u32, s32)
     y = torch.empty_like(r)
     new_state = torch.empty_like(s32)
     flags = _lib.FLOOR_DECAY if T > 1 else 0
-    fn, wsq = (L.wkv5_forward, L.wkv5_forward_workspace) if version == 5 else (L.wkv6_forward, L.wkv6_forward_workspace)
-    nws = wsq(B, T, C, H, dt, _algo)
-    ws = _workspace(nws, r.device)
-    check(fn(_stream(), B, T, C, H, dt, flags, _algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
-             _ptr(y), _ptr(new_state), _ptr(ws), ws.numel()), f"wkv{version}_forward")
-    return y, new_state
+    algo = _algo
+    fn, fq, bq = (L.wkv5_forward, L.wkv5_forward_workspace, L.wkv5_backward_workspace) if version == 5 else \
+                 (L.wkv6_forward, L.wkv6_forward_workspace, L.wkv6_backward_workspace)
+    ws = None
+    if need_grad and fq(B, T, C, H, dt, algo) > 0:
+        ws = _workspace(max(fq(B, T, C, H, dt, algo), bq(B, T, C, H, dt, algo)), r.device)
+    check(fn(_stream(), B, T, C, H, dt, flags, algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
+             _ptr(y), _ptr(new_state), _ptr(ws), 0 if ws is None else ws.numel()), f"wkv{version}_forward")
+    return y, new_state, ws, algo
 
 
-def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate):
+def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate, ws, algo):
     L = _lib.lib()
     dt = _DT[r.dtype]
     gr, gk, gv = torch.empty_like(r), torch.empty_like(k), torch.empty_like(v)
@@ -88,8 +94,11 @@ def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate):
     gs = torch.empty_like(s32)
     flags = _lib.FLOOR_DECAY if T > 1 else 0
     fn, wsq = (L.wkv5_backward, L.wkv5_backward_workspace) if version == 5 else (L.wkv6_backward, L.wkv6_backward_workspace)
-    ws = _workspace(wsq(B, T, C, H, dt, _algo), r.device)
-    check(fn(_stream(), B, T, C, H, dt, flags, _algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
+    if ws is not None:
+        flags |= _lib.CHECKPOINTS_VALID
+    else:
+        ws = _workspace(wsq(B, T, C, H, dt, algo), r.device)
+    check(fn(_stream(), B, T, C, H, dt, flags, algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
              _ptr(gy), _ptr(gstate), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs), _ptr(ws), ws.numel()),
           f"wkv{version}_backward")
     return gr, gk, gv, gw, gu, gs
@@ -106,10 +115,12 @@ class WKV_5(torch.autograd.Function):
         assert state.shape == (B, H, HEAD, HEAD) and H * HEAD == C
         u32 = u.float().contiguous().view(H, HEAD)
         w32 = w.view(H, HEAD)
+        need_grad = any(t.requires_grad for t in (state, r, k, v, w, u))
         with torch.no_grad():
-            y, new_state = _forward56(5, B, T, C, H, r, k, v, w32, u32, state)
+            y, new_state, ws, algo = _forward56(5, B, T, C, H, r, k, v, w32, u32, state, need_grad)
         ctx.dims = (B, T, C, H)
         ctx.meta = (w.shape, u.shape, u.dtype)
+        ctx.ws, ctx.algo = ws, algo
         ctx.save_for_backward(r, k, v, w32, u32, state)
         return y, new_state
 
@@ -122,7 +133,7 @@ class WKV_5(torch.autograd.Function):
         assert gy.dtype == r.dtype
         gstate = None if gstate is None else gstate.float().contiguous()
         with torch.no_grad():
-            gr, gk, gv, gw, gu, gs = _backward56(5, B, T, C, H, r, k, v, w32, u32, state, gy, gstate)
+            gr, gk, gv, gw, gu, gs = _backward56(5, B, T, C, H, r, k, v, w32, u32, state, gy, gstate, ctx.ws, ctx.algo)
         return (None, None, None, None, gs, gr, gk, gv, gw.view(wshape), gu.view(ushape).to(udtype))
 
 
@@ -137,10 +148,12 @@ class WKV_6(torch.autograd.Function):
         u32 = u.float().contiguous().view(H, HEAD)
         w32 = w.float()
         s32 = s.float()
+        need_grad = any(t.requires_grad for t in (r, k, v, w, u, s))
         with torch.no_grad():
-            y, new_state = _forward56(6, B, T, C, H, r, k, v, w32, u32, s32)
+            y, new_state, ws, algo = _forward56(6, B, T, C, H, r, k, v, w32, u32, s32, need_grad)
         ctx.dims = (B, T, C, H)
         ctx.meta = (w.dtype, u.shape, u.dtype, s.dtype)
+        ctx.ws, ctx.algo = ws, algo
         ctx.save_for_backward(r, k, v, w32, u32, s32)
         return y, new_state.to(s.dtype)
 
@@ -153,7 +166,7 @@ class WKV_6(torch.autograd.Function):
         assert gy.dtype == r.dtype
         gstate = None if gstate is None else gstate.float().contiguous()
         with torch.no_grad():
-            gr, gk, gv, gw, gu, gs = _backward56(6, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate)
+            gr, gk, gv, gw, gu, gs = _backward56(6, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate, ctx.ws, ctx.algo)
         return (None, None, None, None, gr, gk, gv, gw.to(wdtype), gu.view(ushape).to(udtype), gs.to(sdtype))
 
 

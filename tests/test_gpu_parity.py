@@ -235,3 +235,117 @@ def test_cumsum_decay_helper(chunk):
     w5 = O.decay_from_raw(raw[0, 0]).view(1, H, 1, K).expand(1, H, T, K)
     tab5 = O.cumsum_decay(w5, chunk, 64)
     assert_close(out5["incl"], tab5.incl.reshape(1, H, T, K).transpose(1, 2).reshape(1, T, C), 1e-5, "incl v5")
+
+
+# ------------------------------------------------- blocked matrix-core path --
+def run_gpu56_forward(version, wl, algo):
+    import rwkv_wkv_hip as W
+    W.set_algo(algo)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.to(dev()) for n, x in wl.tensors.items()}
+    with torch.no_grad():
+        if version == 5:
+            y, s = W.WKV_5.apply(B, T, C, H, g["state"], g["r"], g["k"], g["v"], g["w"], g["u"])
+        else:
+            y, s = W.WKV_6.apply(B, T, C, H, g["r"], g["k"], g["v"], g["w"], g["u"], g["state"])
+    torch.cuda.synchronize()
+    W.set_algo("auto")
+    return y, s
+
+
+@pytest.mark.parametrize("version", [5, 6])
+@pytest.mark.parametrize("T", [1, 16, 50, 64, 128, 200, 512])
+def test_chunked_forward_matches_oracle(version, T):
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=2, T=T, C=192, H=3, dtype=torch.bfloat16)
+    print(f"case chunked fwd v{version} T={T}", flush=True)
+    y, s = run_gpu56_forward(version, wl, "chunked")
+    t = wl.tensors
+    with torch.no_grad():
+        if version == 5:
+            y_ref, s_ref = O.wkv5_op(wl.B, T, wl.C, wl.H, t["state"], t["r"], t["k"], t["v"], t["w"], t["u"])
+        else:
+            y_ref, s_ref = O.wkv6_op(wl.B, T, wl.C, wl.H, t["r"], t["k"], t["v"], t["w"], t["u"], t["state"])
+    assert_close(y, y_ref, 2e-2, "y")
+    assert_close(s, s_ref, 2e-2, "state")
+    # and against the per-token fp32 kernel on the same device
+    y2, s2 = run_gpu56_forward(version, wl, "recurrent")
+    assert_close(y, y2, 2e-2, "y vs recurrent")
+    assert_close(s, s2, 2e-2, "state vs recurrent")
+
+
+def test_chunked_forward_strong_decay_and_floor():
+    """Decays at and below the floor for whole blocks: the re-centred factors
+    reach e^{+-42} and must neither overflow nor lose the result."""
+    from rwkv_wkv_hip import configs
+    wl = configs.make(3, B=1, T=128, C=128, H=2, dtype=torch.bfloat16)
+    w = wl.tensors["w"]
+    w[:, :, :32] = 1.9            # exp(-exp(1.9)) = 1.2e-3 < 0.005 -> floored
+    w[:, :, 32:64] = 1.6          # exp(-exp(1.6)) = 7.1e-3, just above the floor
+    w[:, 40:60, 64:96] = 5.0
+    y, s = run_gpu56_forward(6, wl, "chunked")
+    t = wl.tensors
+    with torch.no_grad():
+        y_ref, s_ref = O.wkv6_op(wl.B, wl.T, wl.C, wl.H, t["r"], t["k"], t["v"], t["w"], t["u"], t["state"])
+    assert_close(y, y_ref, 2e-2, "y")
+    assert_close(s, s_ref, 2e-2, "state")
+
+
+@pytest.mark.parametrize("version", [5, 6])
+@pytest.mark.parametrize("T", [16, 40, 64, 128, 200, 512])
+def test_chunked_forward_backward_matches_oracle(version, T):
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=2, T=T, C=192, H=3, dtype=torch.bfloat16)
+    print(f"case chunked fwd+bwd v{version} T={T}", flush=True)
+    got = run_gpu56(version, wl, algo="chunked")
+    ref = run_oracle56(version, wl)
+    compare(got, ref, 2e-2, f"chunked v{version}/T{T}")
+
+
+@pytest.mark.parametrize("version", [5, 6])
+def test_chunked_truncated_bptt_and_floor(version):
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=1, T=192, C=128, H=2, dtype=torch.bfloat16)
+    w = wl.tensors["w"]
+    if version == 5:
+        w[0, 3] = 2.5
+        w[1, 17] = 1.8
+    else:
+        w[0, 5, 3] = 2.5
+        w[0, 100:140, 64:96] = 1.9
+    got = run_gpu56(version, wl, with_gstate=False, algo="chunked")
+    ref = run_oracle56(version, wl, with_gstate=False)
+    compare(got, ref, 2e-2, f"chunked trunc/floor v{version}")
+    gw = got["gw"].cpu()
+    if version == 5:
+        assert gw[0, 3] == 0 and gw[1, 17] == 0 and gw[0, 4] != 0
+    else:
+        assert gw[0, 5, 3] == 0 and (gw[0, 100:140, 64:96] == 0).all() and gw[0, 5, 4] != 0
+
+
+def test_chunked_backward_rebuilds_checkpoints_when_not_given():
+    """Backward through the C ABI without WKV_CHECKPOINTS_VALID equals backward with it."""
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    wl = configs.make(3, B=1, T=256, C=128, H=2, dtype=torch.bfloat16)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.to(dev()).contiguous() for n, x in wl.tensors.items()}
+    p = lambda x: x.data_ptr()
+    outs = []
+    for valid in (True, False):
+        ws = torch.zeros(L.wkv6_backward_workspace(B, T, C, H, 1, 2), dtype=torch.uint8, device=dev())
+        y, so = torch.empty_like(g["r"]), torch.empty_like(g["state"])
+        flags = _lib.FLOOR_DECAY
+        if valid:
+            assert L.wkv6_forward(None, B, T, C, H, 1, flags, 2, p(g["r"]), p(g["k"]), p(g["v"]), p(g["w"]), p(g["u"]),
+                                  p(g["state"]), p(y), p(so), p(ws), ws.numel()) == 0
+            flags |= _lib.CHECKPOINTS_VALID
+        gr, gk, gv = (torch.empty_like(g["r"]) for _ in range(3))
+        gw, gu, gs = torch.empty_like(g["w"]), torch.empty_like(g["u"]), torch.empty_like(g["state"])
+        assert L.wkv6_backward(None, B, T, C, H, 1, flags, 2, p(g["r"]), p(g["k"]), p(g["v"]), p(g["w"]), p(g["u"]),
+                               p(g["state"]), p(g["dy"]), p(g["dstate"]), p(gr), p(gk), p(gv), p(gw), p(gu), p(gs),
+                               p(ws), ws.numel()) == 0
+        torch.cuda.synchronize()
+        outs.append((gr, gk, gv, gw, gu, gs))
+    for a, b_ in zip(*outs):
+        assert torch.equal(a, b_)
