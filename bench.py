@@ -35,6 +35,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline times")
     ap.add_argument("--rotate", type=int, default=3, help="distinct input sets cycled through")
+    ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
     return ap.parse_args()
 
 
@@ -226,6 +227,7 @@ def main():
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     runner = (Runner4 if a.cfg == 2 else Runner56)(a.cfg, a.algo, a.rotate)
+    assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
     for _ in range(a.warmup):
         runner.step()
@@ -262,7 +264,7 @@ def main():
            "value": tok_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": runner.dtype_name, "data": "synthetic",
-           "config": {"workload": runner.desc, "algo": a.algo},
+           "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto"},
            "roofline": roofline}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(a.cfg, a.cpu_heads)

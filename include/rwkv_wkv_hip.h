@@ -56,6 +56,13 @@ typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
 const char *wkv_strerror(int status);
 int wkv_abi_version(void);
 
+/* Tuning knobs (no counterpart in the reference).  WKV_TUNE_SEGMENTS: number of
+ * time segments one (batch, head) sequence is cut into by the chunked algorithm
+ * so that short batches still fill the GPU; 0 = choose from the shape (default),
+ * 1..64 = force.  Results do not depend on it beyond fp32 rounding order. */
+#define WKV_TUNE_SEGMENTS 1
+int wkv_tune(int key, int value);
+
 /* Timing hook for benchmarks (no counterpart in the reference).
  * wkv_profile_begin: from now on the first `max_launches` launches of the
  * kernel `kernel_id` are bracketed by HIP events recorded on the stream the

@@ -45,14 +45,12 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
     if (a < 0) return a;
     if (a == WKV_ALGO_CHUNKED) {
         // with a workspace the state at the start of every 64-token step is left there for backward
-        float *ckpt = nullptr;
         if (workspace) {
             if (!aligned16(workspace)) return WKV_ERR_ALIGN;
-            if (workspace_bytes < chunked::checkpoint_bytes(B, T, H)) return WKV_ERR_WORKSPACE;
-            ckpt = (float *)workspace;
+            if (workspace_bytes < chunked::forward_workspace(B, T, H)) return WKV_ERR_WORKSPACE;
         }
         hipError_t e = chunked::forward_launch((hipStream_t)stream, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
-                                               state_out, ckpt, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+                                               state_out, workspace, true, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
         return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
     }
     hipError_t e = recurrent_forward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
@@ -62,7 +60,7 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
 
 size_t forward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
     if (check_dims56(B, T, C, H, dtype)) return 0;
-    return pick_algo56(algo, T, dtype, false) == WKV_ALGO_CHUNKED ? chunked::checkpoint_bytes(B, T, H) : 0;
+    return pick_algo56(algo, T, dtype, false) == WKV_ALGO_CHUNKED ? chunked::forward_workspace(B, T, H) : 0;
 }
 
 size_t backward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
@@ -124,6 +122,15 @@ const char *wkv_strerror(int status) {
 }
 
 int wkv_abi_version(void) { return 1; }
+
+int wkv_tune(int key, int value) {
+    if (key == WKV_TUNE_SEGMENTS) {
+        if (value < 0 || value > chunked::MAX_SEG) return WKV_ERR_DIMS;
+        chunked::forced_segments() = value;
+        return WKV_OK;
+    }
+    return WKV_ERR_DIMS;
+}
 
 int wkv_profile_begin(int kernel_id, int max_launches) {
     ProfileSlot &p = profile_slot();

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <vector>
+#include <algorithm>
+#include <cstdlib>
 
 namespace wkv {
 

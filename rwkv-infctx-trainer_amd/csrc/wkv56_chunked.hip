@@ -125,29 +125,58 @@ struct FwdTiles {
     float rho[SB];           // r . (u o k) per token
 };
 
-// Forward over tokens [0, Tlen) of one (batch, head).  ckpt (optional) receives
-// the state at the start of every 64-token step, [bh][step][key][value] fp32.
-template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
+// One segment's summary for the time-parallel split: what the segment does to a
+// state handed in, S_out = decay o S_in + delta (forward), or to a state gradient
+// handed back (backward).  [key][value] fp32 plus one decay per key.
+constexpr int PART = HEAD * HEAD + HEAD;
+
+// Forward over one segment (`sps` 64-token steps) of one (batch, head); grid =
+// B*H*nseg.  The sequence is cut into nseg segments that run in parallel:
+//   STATE_ONLY pass  (segments 0..nseg-2): from a zero state, leaves the segment's
+//                    summary in `part`;
+//   main pass        (all segments): folds the summaries of the earlier segments
+//                    into s_in to get its own starting state, then produces y.
+// ckpt (optional) receives the state at the start of every 64-token step,
+// [bh][step][key][value] fp32; the last segment writes s_out.
+template <bool PER_TOKEN_W, bool STATE_ONLY>
+__global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, int sps,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
-        bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, int floor_decay)
+        bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, float *__restrict__ part,
+        int floor_decay)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     FwdTiles &sm = *reinterpret_cast<FwdTiles *>(smem_raw);
-    const int bh = blockIdx.x, b = bh / H, h = bh % H;
+    const int nsegk = STATE_ONLY ? nseg - 1 : nseg;
+    const int bh = blockIdx.x / nsegk, seg = blockIdx.x % nsegk, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
+    const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
 
     // state tiles: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]
-    f4 S[4];
-    {
+    f4 S[4], Dacc[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+        S[kk] = f4{0.f, 0.f, 0.f, 0.f};
+        Dacc[kk] = f4{1.f, 1.f, 1.f, 1.f};
+    }
+    if (!STATE_ONLY) {
         const float *sp = s_in + (size_t)bh * HEAD * HEAD;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
             for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
+        for (int gg = 0; gg < seg; gg++) {           // states of the earlier segments, in order
+            const float *pp = part + ((size_t)bh * nseg + gg) * PART;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int row = 16 * kk + 4 * g + e;
+                    S[kk][e] = fmaf(pp[HEAD * HEAD + row], S[kk][e], pp[row * HEAD + 16 * wv + n]);
+                }
+        }
     }
     // staging role: block wv of the step, tokens 8*half..8*half+7 of it, channels c0, c0+1
     const int half = lane >> 5, c0 = 2 * (lane & 31);
@@ -177,8 +206,8 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
         }
     };
 
-    fetch(0);
-    for (int sb = 0; sb < nsb; sb++) {
+    fetch(sb0);
+    for (int sb = sb0; sb < sb1; sb++) {
         // ---------------- prepare the scaled operands of 64 tokens
         {
             float ia[8], ib[8], la[8], lb[8];
@@ -207,15 +236,17 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
                 const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
                 const int o = (16 * wv + 8 * half + x) * LD + c0;
                 uint32_t hi, lo;
-                split2(rha, rhb, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
-                split2(rha * ea_nm, rhb * eb_nm, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.rd[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.rdl[o]) = lo;
-                split2(kha * ea_mb, khb * eb_mb, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.kd[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.kdl[o]) = lo;
+                if (!STATE_ONLY) {
+                    split2(rha, rhb, hi, lo);
+                    *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
+                    *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
+                    split2(rha * ea_nm, rhb * eb_nm, hi, lo);
+                    *reinterpret_cast<uint32_t *>(&sm.rd[o]) = hi;
+                    *reinterpret_cast<uint32_t *>(&sm.rdl[o]) = lo;
+                    split2(kha * ea_mb, khb * eb_mb, hi, lo);
+                    *reinterpret_cast<uint32_t *>(&sm.kd[o]) = hi;
+                    *reinterpret_cast<uint32_t *>(&sm.kdl[o]) = lo;
+                }
                 p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
                 split2(kha, khb, hi, lo);
                 gk_h.add(x, hi);
@@ -227,14 +258,16 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
             gk_l.put(sm.khTl, ot);
             gv_.put(sm.vT, ot);
             if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(tota), __expf(totb));
-            const float tot_p = sum8_over_half(p, lane);
-            if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
+            if (!STATE_ONLY) {
+                const float tot_p = sum8_over_half(p, lane);
+                if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
+            }
         }
         __syncthreads();
-        if (sb + 1 < nsb) fetch(sb + 1);          // next step's loads fly during the MFMA phase
+        if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
 
         // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
-        if (ckpt) {
+        if (!STATE_ONLY && ckpt) {
             float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD;
 #pragma unroll
             for (int kk = 0; kk < 4; kk++)
@@ -244,6 +277,8 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             if (sb * SB + 16 * q >= Tlen) break;
+            const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
+            if (!STATE_ONLY) {
             // A^T[s][t] = sum_i kd[s][i] rd[t][i]; lane gets s = 4g+e, t = n
             // (operands carried as bf16 head + remainder; head*head + rem*head + head*rem)
             f4 at = {0.f, 0.f, 0.f, 0.f};
@@ -264,7 +299,6 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
             }
             s4 a_hi, a_lo;                                  // A[t = n][s = 4g..4g+3]
             split4(at, a_hi, a_lo);
-            const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
             f4 yt = {0.f, 0.f, 0.f, 0.f};
             yt = mma2(a_hi, a_lo, v_op, v_op, yt);
 #pragma unroll
@@ -283,17 +317,29 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H,
                 const int t = sb * SB + 16 * q + 4 * g + e;
                 if (y && t < Tlen) y[base + (size_t)t * C + 16 * wv + n] = bf16{bf16_bits(yt[e])};
             }
+            }
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) {
                 const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
                 S[kk][0] *= d4.x; S[kk][1] *= d4.y; S[kk][2] *= d4.z; S[kk][3] *= d4.w;
+                if (STATE_ONLY) { Dacc[kk][0] *= d4.x; Dacc[kk][1] *= d4.y; Dacc[kk][2] *= d4.z; Dacc[kk][3] *= d4.w; }
                 S[kk] = mma2(frag(sm.khT, 16 * kk + n, 16 * q + 4 * g), frag(sm.khTl, 16 * kk + n, 16 * q + 4 * g),
                              v_op, v_op, S[kk]);
             }
         }
         __syncthreads();
     }
-    if (s_out) {
+    if (STATE_ONLY) {
+        float *pp = part + ((size_t)bh * nseg + seg) * PART;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int row = 16 * kk + 4 * g + e;
+                pp[row * HEAD + 16 * wv + n] = S[kk][e];
+                if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
+            }
+    } else if (s_out && seg == nseg - 1) {
         float *op = s_out + (size_t)bh * HEAD * HEAD;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
@@ -348,19 +394,20 @@ __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane g
 }
 
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
+__global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H, int nseg, int sps,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
-        const float *__restrict__ gs_out, const float *__restrict__ ckpt,
+        const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
         bf16 *__restrict__ gr, bf16 *__restrict__ gk, bf16 *__restrict__ gv, float *__restrict__ gw_tok,
         float *__restrict__ gw_part, float *__restrict__ gu_part, float *__restrict__ gs_in, int floor_decay)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     BwdTiles &sm = *reinterpret_cast<BwdTiles *>(smem_raw);
-    const int bh = blockIdx.x, b = bh / H, h = bh % H;
+    const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
+    const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
     const int own = 16 * wv + n;                 // key channel (gr, gk, gw) / value channel (gv) of this lane
     const float u_i = u[h * HEAD + own];
 
@@ -375,6 +422,18 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
                 GT[kk][e] = gp ? gp[own * HEAD + 16 * kk + 4 * g + e] : 0.f;
                 GJ[kk][e] = gp ? gp[(16 * kk + 4 * g + e) * HEAD + own] : 0.f;
             }
+        for (int gg = nseg - 1; gg > seg; gg--) {      // gradients through the later segments, last first
+            const float *pp = gpart + ((size_t)bh * nseg + gg) * PART;
+            const float d_own = pp[HEAD * HEAD + own];
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int x = 16 * kk + 4 * g + e;
+                    GT[kk][e] = fmaf(d_own, GT[kk][e], pp[own * HEAD + x]);
+                    GJ[kk][e] = fmaf(pp[HEAD * HEAD + x], GJ[kk][e], pp[x * HEAD + own]);
+                }
+        }
     }
     float A_run = 0.f, gu_acc = 0.f, gw_acc = 0.f;
 
@@ -406,8 +465,8 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
         }
     };
 
-    fetch(nsb - 1);
-    for (int sb = nsb - 1; sb >= 0; sb--) {
+    fetch(sb1 - 1);
+    for (int sb = sb1 - 1; sb >= sb0; sb--) {
         // ---------------- prepare the operands of 64 tokens
         {
             float ia[8], ib[8], la[8], lb[8];
@@ -473,7 +532,7 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
             if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
         }
         __syncthreads();
-        if (sb > 0) fetch(sb - 1);
+        if (sb > sb0) fetch(sb - 1);
 
         // ---------------- rebuild the state at the start of each block (value-major slice: key `own`)
         f4 ST[4];
@@ -653,7 +712,7 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
         __syncthreads();
     }
 
-    if (gs_in) {
+    if (gs_in && seg == 0) {
         float *gp = gs_in + (size_t)bh * HEAD * HEAD + own * HEAD;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
@@ -661,48 +720,200 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H,
     }
     gu_acc = group_sum4(gu_acc);
     gw_acc = group_sum4(gw_acc);
-    if (g == 0) {
-        gu_part[(size_t)bh * HEAD + own] = gu_acc;
+    if (g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
+        const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
+        gu_part[po] = gu_acc;
         if (!PER_TOKEN_W) {
             bool fl;
             const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
-            gw_part[(size_t)bh * HEAD + own] = fl ? 0.f : gw_acc * l;
+            gw_part[po] = fl ? 0.f : gw_acc * l;
         }
     }
+}
+
+// State-gradient summary of one segment (segments 1..nseg-1) for the backward
+// split: from a zero gradient, walks the segment's tokens last to first with
+//   G <- e^{b} o G + (r e^{excl})^T gy      per 16-token block
+// and leaves  delta = G, decay = product of e^{b}  in gpart.  One wavefront per
+// 16 value columns, as the forward's state.
+struct GPassTiles {
+    uint16_t rhT[SB * LD];   // r e^{excl}   [key][token]  head / remainder
+    uint16_t rhTl[SB * LD];
+    uint16_t gyT[SB * LD];   // gy           [value][token]
+    float dec[4][HEAD];
+};
+
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(NT) void gradient_pass(int Tlen, int C, int H, int nseg, int sps,
+        const bf16 *__restrict__ r, const float *__restrict__ wraw, const bf16 *__restrict__ gy,
+        float *__restrict__ gpart, int floor_decay)
+{
+    __shared__ __align__(16) GPassTiles sm;
+    const int bh = blockIdx.x / (nseg - 1), seg = 1 + blockIdx.x % (nseg - 1), b = bh / H, h = bh % H;
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    const int nsb = (Tlen + SB - 1) / SB;
+    const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
+    const int half = lane >> 5, c0 = 2 * (lane & 31);
+    float2 l_const = make_float2(0.f, 0.f);
+    if (!PER_TOKEN_W) {
+        l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
+        l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
+    }
+    f4 G[4], Dacc[4];           // G[kk][e] = G[key 16kk+4g+e][value 16wv+n]
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+        G[kk] = f4{0.f, 0.f, 0.f, 0.f};
+        Dacc[kk] = f4{1.f, 1.f, 1.f, 1.f};
+    }
+    uint32_t pr[8], pg[8];
+    float2 pw[8];
+    auto fetch = [&](int sb) {
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+            const int t = sb * SB + 16 * wv + 8 * half + x;
+            if (t < Tlen) {
+                const size_t o = base + (size_t)t * C + c0;
+                pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
+                pg[x] = *reinterpret_cast<const uint32_t *>(gy + o);
+                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
+            } else {
+                pr[x] = pg[x] = 0;
+                pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);
+            }
+        }
+    };
+    fetch(sb1 - 1);
+    for (int sb = sb1 - 1; sb >= sb0; sb--) {
+        {
+            float ea[8], eb[8];                 // exclusive running log decay inside this lane's 8 tokens
+            float ra = 0.f, rb = 0.f;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                ea[x] = ra; eb[x] = rb;
+                ra += PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
+                rb += PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
+            }
+            const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
+            const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
+            Gather8 gr_h, gr_l, gg_;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                uint32_t hi, lo;
+                split2(bf_lo(pr[x]) * __expf(ea[x] + offa), bf_hi(pr[x]) * __expf(eb[x] + offb), hi, lo);
+                gr_h.add(x, hi);
+                gr_l.add(x, lo);
+                gg_.add(x, pg[x]);
+            }
+            const int ot = c0 * LD + 16 * wv + 8 * half;
+            gr_h.put(sm.rhT, ot);
+            gr_l.put(sm.rhTl, ot);
+            gg_.put(sm.gyT, ot);
+            if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(ra + oa), __expf(rb + ob));
+        }
+        __syncthreads();
+        if (sb > sb0) fetch(sb - 1);
+#pragma unroll
+        for (int q = 3; q >= 0; q--) {
+            if (sb * SB + 16 * q >= Tlen) continue;
+            const s4 gyTf = frag(sm.gyT, 16 * wv + n, 16 * q + 4 * g);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
+                G[kk][0] *= d4.x; G[kk][1] *= d4.y; G[kk][2] *= d4.z; G[kk][3] *= d4.w;
+                Dacc[kk][0] *= d4.x; Dacc[kk][1] *= d4.y; Dacc[kk][2] *= d4.z; Dacc[kk][3] *= d4.w;
+                G[kk] = mma2(frag(sm.rhT, 16 * kk + n, 16 * q + 4 * g), frag(sm.rhTl, 16 * kk + n, 16 * q + 4 * g),
+                             gyTf, gyTf, G[kk]);
+            }
+        }
+        __syncthreads();
+    }
+    float *pp = gpart + ((size_t)bh * nseg + seg) * PART;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int row = 16 * kk + 4 * g + e;
+            pp[row * HEAD + 16 * wv + n] = G[kk][e];
+            if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
+        }
 }
 
 size_t checkpoint_bytes(int B, int Tlen, int H) {
     return (size_t)B * H * ((Tlen + SB - 1) / SB) * HEAD * HEAD * sizeof(float);
 }
 
+// How many time segments run in parallel for one (batch, head): enough workgroups
+// to give every CU about two, each segment at least four 64-token steps long.
+// RWKV_WKV_NSEG overrides it (tuning aid).
+struct SegPlan { int nseg, sps; };
+inline int &forced_segments() {          // 0 = choose automatically (wkv_tune)
+    static int v = [] { const char *e = getenv("RWKV_WKV_NSEG"); return e ? atoi(e) : 0; }();
+    return v;
+}
+static SegPlan plan_segments(int BH, int Tlen) {
+    const int nsb = (Tlen + SB - 1) / SB;
+    const int forced = forced_segments();
+    int want = forced > 0 ? forced : (512 + BH - 1) / BH;
+    want = std::max(1, std::min(want, forced > 0 ? nsb : std::max(1, nsb / 4)));
+    const int sps = (nsb + want - 1) / want;
+    return SegPlan{(nsb + sps - 1) / sps, sps};
+}
+constexpr int MAX_SEG = 64;
+static size_t part_bytes(int B, int H) { return (size_t)B * H * MAX_SEG * PART * sizeof(float); }
+
+// workspace of a forward call: checkpoints | forward segment summaries
+size_t forward_workspace(int B, int Tlen, int H) { return checkpoint_bytes(B, Tlen, H) + part_bytes(B, H); }
+// workspace of a backward call: the forward's | backward segment summaries | gu, gw partials (B*MAX_SEG, C)
+size_t backward_workspace(int B, int Tlen, int C, int H) {
+    return forward_workspace(B, Tlen, H) + part_bytes(B, H) + 2 * (size_t)B * MAX_SEG * C * sizeof(float);
+}
+
+template <class K>
+static hipError_t allow_lds(K kernel, size_t bytes) {
+    return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+// workspace == nullptr: single segment, no checkpoints kept
 hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
                           const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
-                          float *ckpt, int floor_decay) {
+                          void *workspace, bool keep_ckpt, int floor_decay) {
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)forward<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)sizeof(FwdTiles));
-        if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute((const void *)forward<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)sizeof(FwdTiles));
+        hipError_t e = allow_lds(forward<true, false>, sizeof(FwdTiles));
+        if (e == hipSuccess) e = allow_lds(forward<false, false>, sizeof(FwdTiles));
+        if (e == hipSuccess) e = allow_lds(forward<true, true>, sizeof(FwdTiles));
+        if (e == hipSuccess) e = allow_lds(forward<false, true>, sizeof(FwdTiles));
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    dim3 grid(B * H), block(NT);
+    SegPlan pl = workspace ? plan_segments(B * H, Tlen) : SegPlan{1, (Tlen + SB - 1) / SB};
+    if (pl.nseg > MAX_SEG) pl = SegPlan{1, (Tlen + SB - 1) / SB};
+    float *ckpt = (workspace && keep_ckpt) ? (float *)workspace : nullptr;
+    float *part = workspace ? (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H)) : nullptr;
+    const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v;
+    dim3 block(NT);
+    if (pl.nseg > 1) {
+        dim3 grid(B * H * (pl.nseg - 1));
+        if (per_token)
+            hipLaunchKernelGGL((forward<true, true>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk,
+                               vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part, floor_decay);
+        else
+            hipLaunchKernelGGL((forward<false, true>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr,
+                               kk, vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part, floor_decay);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    dim3 grid(B * H * pl.nseg);
     prof_begin(KID_CHUNK_FORWARD, s);
     if (per_token)
-        hipLaunchKernelGGL((forward<true>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, (const bf16 *)r, (const bf16 *)k,
-                           (const bf16 *)v, w, u, s_in, (bf16 *)y, s_out, ckpt, floor_decay);
+        hipLaunchKernelGGL((forward<true, false>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv,
+                           w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
     else
-        hipLaunchKernelGGL((forward<false>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, (const bf16 *)r, (const bf16 *)k,
-                           (const bf16 *)v, w, u, s_in, (bf16 *)y, s_out, ckpt, floor_decay);
+        hipLaunchKernelGGL((forward<false, false>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk,
+                           vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
     prof_end(KID_CHUNK_FORWARD, s);
     return hipGetLastError();
-}
-
-// workspace of the backward call: checkpoints | gu partials (B,C) | gw partials (B,C)
-size_t backward_workspace(int B, int Tlen, int C, int H) {
-    return checkpoint_bytes(B, Tlen, H) + 2 * (size_t)B * C * sizeof(float);
 }
 
 hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
@@ -710,37 +921,51 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
                            const float *gs_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gs_in,
                            void *workspace, bool have_ckpt, int floor_decay) {
     float *ckpt = (float *)workspace;
-    float *gu_part = (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H));
-    float *gw_part = gu_part + (size_t)B * C;
+    float *gpart = (float *)((char *)workspace + forward_workspace(B, Tlen, H));
+    float *gu_part = (float *)((char *)gpart + part_bytes(B, H));
+    float *gw_part = gu_part + (size_t)B * MAX_SEG * C;
     if (!have_ckpt) {      // the forward call did not leave its checkpoints here: rebuild them
-        hipError_t e = forward_launch(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, ckpt, floor_decay);
+        hipError_t e = forward_launch(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, workspace,
+                                      true, floor_decay);
         if (e != hipSuccess) return e;
     }
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)backward<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)sizeof(BwdTiles));
-        if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute((const void *)backward<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)sizeof(BwdTiles));
+        hipError_t e = allow_lds(backward<true>, sizeof(BwdTiles));
+        if (e == hipSuccess) e = allow_lds(backward<false>, sizeof(BwdTiles));
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    dim3 grid(B * H), block(NT);
+    SegPlan pl = plan_segments(B * H, Tlen);
+    if (pl.nseg > MAX_SEG) pl = SegPlan{1, (Tlen + SB - 1) / SB};
+    const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v, *gg = (const bf16 *)gy;
+    dim3 block(NT);
+    if (pl.nseg > 1) {
+        dim3 grid(B * H * (pl.nseg - 1));
+        if (per_token)
+            hipLaunchKernelGGL((gradient_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, rr, w, gg, gpart,
+                               floor_decay);
+        else
+            hipLaunchKernelGGL((gradient_pass<false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, rr, w, gg, gpart,
+                               floor_decay);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    dim3 grid(B * H * pl.nseg);
     prof_begin(KID_CHUNK_BACKWARD, s);
     if (per_token)
-        hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, (const bf16 *)r,
-                           (const bf16 *)k, (const bf16 *)v, w, u, (const bf16 *)gy, gs_out, ckpt, (bf16 *)gr,
-                           (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in, floor_decay);
+        hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv, w,
+                           u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in,
+                           floor_decay);
     else
-        hipLaunchKernelGGL((backward<false>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, (const bf16 *)r,
-                           (const bf16 *)k, (const bf16 *)v, w, u, (const bf16 *)gy, gs_out, ckpt, (bf16 *)gr,
-                           (bf16 *)gk, (bf16 *)gv, nullptr, gw_part, gu_part, gs_in, floor_decay);
+        hipLaunchKernelGGL((backward<false>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv, w,
+                           u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr, gw_part,
+                           gu_part, gs_in, floor_decay);
     prof_end(KID_CHUNK_BACKWARD, s);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gu_part, gu);
-    if (!per_token) hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gw_part, gw);
+    hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B * pl.nseg, C, gu_part, gu);
+    if (!per_token) hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B * pl.nseg, C, gw_part, gw);
     return hipGetLastError();
 }
 

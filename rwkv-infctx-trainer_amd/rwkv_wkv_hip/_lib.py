@@ -16,6 +16,7 @@ WKV_F32, WKV_BF16, WKV_F16 = 0, 1, 2
 FLOOR_DECAY = 1
 CHECKPOINTS_VALID = 2
 ALGO_AUTO, ALGO_RECURRENT, ALGO_CHUNKED = 0, 1, 2
+TUNE_SEGMENTS = 1
 
 _P = c_void_p
 _I = c_int
@@ -24,6 +25,7 @@ _I = c_int
 SIGNATURES = {
     "wkv_strerror": (c_char_p, [_I]),
     "wkv_abi_version": (_I, []),
+    "wkv_tune": (_I, [_I, _I]),
     "wkv_profile_begin": (_I, [_I, _I]),
     "wkv_profile_end": (_I, [_P, _I]),
     "wkv6_forward_workspace": (c_size_t, [_I] * 6),

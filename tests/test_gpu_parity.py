@@ -349,3 +349,21 @@ def test_chunked_backward_rebuilds_checkpoints_when_not_given():
         outs.append((gr, gk, gv, gw, gu, gs))
     for a, b_ in zip(*outs):
         assert torch.equal(a, b_)
+
+
+@pytest.mark.parametrize("version", [5, 6])
+@pytest.mark.parametrize("nseg,T", [(1, 1024), (2, 1024), (4, 1024), (3, 1000), (8, 832)])
+def test_chunked_time_segments(version, nseg, T):
+    """The time-parallel split (segment summaries folded in order) gives the same
+    outputs and gradients as the oracle for any number of segments, ragged ones included."""
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    wl = configs.make(1 if version == 5 else 3, B=1, T=T, C=128, H=2, dtype=torch.bfloat16)
+    print(f"case segments v{version} nseg={nseg} T={T}", flush=True)
+    assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg) == 0
+    try:
+        got = run_gpu56(version, wl, algo="chunked")
+    finally:
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, 0) == 0
+    ref = run_oracle56(version, wl)
+    compare(got, ref, 2e-2, f"segments v{version}/n{nseg}/T{T}")
