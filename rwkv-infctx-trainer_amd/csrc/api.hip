@@ -22,10 +22,11 @@ int check_dims56(int B, int T, int C, int H, int dtype) {
     return WKV_OK;
 }
 
-// the blocked matrix-core path takes bf16 streams; everything else goes token by token
-int pick_algo56(int algo, int T, int dtype, bool backward) {
-    (void)backward; (void)T;
-    const bool can_chunk = dtype == WKV_BF16;
+// the blocked matrix-core path takes bf16 streams with the decay floor switched on
+// (whose range analysis relies on the decay floor); everything else goes token by token
+int pick_algo56(int algo, int T, int dtype, unsigned flags) {
+    (void)T;
+    const bool can_chunk = dtype == WKV_BF16 && (flags & WKV_FLOOR_DECAY);
     if (algo == WKV_ALGO_AUTO) return can_chunk ? WKV_ALGO_CHUNKED : WKV_ALGO_RECURRENT;
     if (algo == WKV_ALGO_RECURRENT) return algo;
     if (algo == WKV_ALGO_CHUNKED) return can_chunk ? algo : WKV_ERR_ALGO;
@@ -41,7 +42,7 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
     for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
                           (const void *)state_out})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
-    const int a = pick_algo56(algo, T, dtype, false);
+    const int a = pick_algo56(algo, T, dtype, flags);
     if (a < 0) return a;
     if (a == WKV_ALGO_CHUNKED) {
         // with a workspace the state at the start of every 64-token step is left there for backward
@@ -58,15 +59,18 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
 
+// (sizes are for the larger of the two algorithms a call with these arguments can take)
 size_t forward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
     if (check_dims56(B, T, C, H, dtype)) return 0;
-    return pick_algo56(algo, T, dtype, false) == WKV_ALGO_CHUNKED ? chunked::forward_workspace(B, T, H) : 0;
+    return pick_algo56(algo, T, dtype, WKV_FLOOR_DECAY) == WKV_ALGO_CHUNKED ? chunked::forward_workspace(B, T, H) : 0;
 }
 
 size_t backward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
     if (check_dims56(B, T, C, H, dtype)) return 0;
-    if (pick_algo56(algo, T, dtype, true) == WKV_ALGO_CHUNKED) return chunked::backward_workspace(B, T, C, H);
-    return recurrent_backward_workspace(B, T, C);
+    const size_t rec = recurrent_backward_workspace(B, T, C);
+    if (pick_algo56(algo, T, dtype, WKV_FLOOR_DECAY) == WKV_ALGO_CHUNKED)
+        return std::max(rec, chunked::backward_workspace(B, T, C, H));
+    return rec;
 }
 
 int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
@@ -80,10 +84,12 @@ int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dty
                           (const void *)gstate_out, (const void *)gr, (const void *)gk, (const void *)gv,
                           (const void *)gw, (const void *)gu, (const void *)gstate_in, (const void *)workspace})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
-    const int a = pick_algo56(algo, T, dtype, true);
+    const int a = pick_algo56(algo, T, dtype, flags);
     if (a < 0) return a;
     if (!workspace) return WKV_ERR_NULL;
-    if (workspace_bytes < backward56_workspace(B, T, C, H, dtype, algo)) return WKV_ERR_WORKSPACE;
+    if (workspace_bytes < (a == WKV_ALGO_CHUNKED ? chunked::backward_workspace(B, T, C, H)
+                                                 : recurrent_backward_workspace(B, T, C)))
+        return WKV_ERR_WORKSPACE;
     if (a == WKV_ALGO_CHUNKED) {
         hipError_t e = chunked::backward_launch((hipStream_t)stream, per_token, B, T, C, H, r, k, v, w, u, state_in, gy,
                                                 gstate_out, gr, gk, gv, gw, gu, gstate_in, workspace,

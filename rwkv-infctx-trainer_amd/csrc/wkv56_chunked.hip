@@ -1,40 +1,64 @@
 // WKV5 / WKV6 in blocked form on the matrix cores (bf16 operands, fp32 state).
 //
-// One workgroup of 4 wavefronts per (batch, head) walks the sequence in blocks
-// of 16 tokens.  Inside a block, with incl_t / excl_t the inclusive / exclusive
-// running sums of log w from the block's start, b their total and m = excl_8:
+// A (batch, head) sequence is walked in blocks of 16 tokens.  Inside a block, with
+// incl_t / excl_t the inclusive / exclusive running sums of log w from the block's
+// start and b their total:
 //
-//   y_t = (r_t e^{excl_t}) S  +  sum_{s<t} [(r_t e^{excl_t-m}) . (k_s e^{m-incl_s})] v_s
-//         + (r_t . u k_t) v_t
+//   y_t = (r_t e^{excl_t}) S  +  sum_{s<t} [(r_t e^{excl_t}) . (k_s e^{-incl_s})] v_s  +  (r_t . u k_t) v_t
 //   S  <- e^{b} o S + sum_s (k_s e^{b-incl_s})^T v_s
 //
-// Every exponent above is bounded (|.| <= 8 * 5.3 for the two re-centred
-// factors, <= 0 for the rest, because log w >= ln 0.005), so all factors fit
-// bf16/fp32 without the fp64 the reference needs for its 128-token chunks
-// (RWKV-v5/src/module/rwkv_inner.py:91-93).  The four contractions are
-// 16x16x16 bf16 MFMAs; the state lives in MFMA accumulators for the whole
-// sequence: wavefront w owns value columns 16w..16w+15 of S (all 64 key rows).
+// log w >= ln 0.005, so excl_t >= -79.5 for every token of a block and -incl_s <= 79.5
+// for every s that has a later token in its block: all scaled factors stay inside
+// the bf16/fp32 range without the fp64 the reference needs for its 128-token chunks
+// (RWKV-v5/src/module/rwkv_inner.py:91-93).  The contractions are 16x16x32 bf16
+// MFMAs; the state lives in MFMA accumulators for the whole sequence and enters the
+// next product straight from registers (the accumulator layout of a 16x16 tile is
+// the B-operand layout).
 //
-// The scaled operands are prepared 64 tokens at a time (lane = one channel of
-// one 16-token block: running sum in registers, no cross-lane scan) and laid
-// out in LDS so that every MFMA operand fragment is one 8-byte read; rows are
-// padded to 68 elements, which spreads the 16 rows of a fragment over all banks.
+// Precision: every operand that is not already an exact bf16 input (decay-scaled
+// r and k, the masked intra-block matrices, the state and its gradient) is fed
+// to the matrix cores as a bf16 head plus a bf16 remainder (x ~= hi + lo, 16
+// mantissa bits) and the products hi*hi + lo*hi + hi*lo are accumulated in fp32,
+// two 16-deep products per 16x16x32 instruction.  This is what keeps the decay
+// gradient, a difference of large running sums, at fp32-like accuracy.
+//
+// The scaled operands are prepared 64 tokens at a time (a lane keeps the running
+// log decay of its tokens in registers; one or two shuffles join the pieces of a
+// block) and laid out in LDS so that every MFMA operand fragment is one 8-byte
+// read; rows are padded to 68 elements, which spreads the 16 rows of a fragment
+// over all banks.
+//
+// Time-parallel split: a sequence is cut into segments that run as separate
+// workgroups; a light pass leaves each segment's effect on a state handed in
+// (S_out = decay o S_in + delta), the main pass folds the earlier segments'
+// summaries in order.  Backward does the same with the state gradient.
 #include "common.h"
 
 namespace wkv {
 namespace chunked {
 
+// optional per-phase cycle counts of workgroup 0 (development aid, off by default)
+#ifdef WKV_PHASE_TIMING
+#define PT_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}; long long pt_last_ = clock64();
+#define PT_MARK(i) { const long long now_ = clock64(); pt_[i] += now_ - pt_last_; pt_last_ = now_; }
+#define PT_PRINT(name) if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) printf("%s[%d]: stage %lld sync %lld compute %lld sync %lld other %lld aux %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5]);
+#else
+#define PT_DECL
+#define PT_MARK(i)
+#define PT_PRINT(name)
+#endif
+
 typedef short s4 __attribute__((ext_vector_type(4)));
+typedef short s8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
 constexpr int SB = 64;        // tokens prepared per staging step
 constexpr int LD = 68;        // padded row length of a 64x64 bf16 tile in LDS
-constexpr int NT = 256;
+constexpr int NT_F = 256;     // forward: 4 wavefronts
+constexpr int NT_B = 512;     // backward: 8 wavefronts (4 key-side + 4 value-side)
 
-typedef short s8 __attribute__((ext_vector_type(8)));
-typedef __bf16 b8 __attribute__((ext_vector_type(8)));
-
-// D[m][n] += sum_k A[m][k] B[k][n] for one 16-deep product.  Issued as a 16x16x32 MFMA
+// One 16-deep product, D[m][n] += sum_k A[m][k] B[k][n].  Issued as a 16x16x32 MFMA
 // with a zero upper half: on gfx950 a 16x16x16 MFMA chained on the accumulator of a
 // 16x16x32 one returned corrupted rows in this kernel, and both cost one issue slot.
 __device__ __forceinline__ f4 mma(s4 a, s4 b, f4 c) {
@@ -59,7 +83,6 @@ __device__ __forceinline__ s4 as_s4(uint32_t a, uint32_t b) {
     const uint2 x = make_uint2(a, b);
     return __builtin_bit_cast(s4, x);
 }
-__device__ __forceinline__ s4 pack(f4 x) { return as_s4(bf16_pack2(x[0], x[1]), bf16_pack2(x[2], x[3])); }
 // x ~= hi + lo with both parts bf16: 16 mantissa bits instead of 8
 __device__ __forceinline__ void split2(float a, float b, uint32_t &hi, uint32_t &lo) {
     hi = bf16_pack2(a, b);
@@ -71,6 +94,11 @@ __device__ __forceinline__ void split4(f4 x, s4 &hi, s4 &lo) {
     split2(x[2], x[3], h1, l1);
     hi = as_s4(h0, h1);
     lo = as_s4(l0, l1);
+}
+__device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane groups of 16
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
 }
 
 // sum each of 8 per-lane values over the 32 lanes of a half wavefront; afterwards
@@ -95,34 +123,37 @@ __device__ __forceinline__ float sum8_over_half(const float (&p)[8], int lane) {
     return x;
 }
 __device__ __forceinline__ int sum8_index(int lane) { return ((lane >> 4) & 1) * 4 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1); }
+// the same for 4 values over 16 lanes: lane L ends with the total of index 2*b3 + b2
+__device__ __forceinline__ float sum4_over_16(const float (&p)[4], int lane) {
+    float a2[2];
+    const bool h3 = lane & 8, h2 = lane & 4;
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        const float keep = h3 ? p[e + 2] : p[e], send = h3 ? p[e] : p[e + 2];
+        a2[e] = keep + __shfl_xor(send, 8);
+    }
+    const float keep = h2 ? a2[1] : a2[0], send = h2 ? a2[0] : a2[1];
+    float x = keep + __shfl_xor(send, 4);
+    x += __shfl_xor(x, 2);
+    x += __shfl_xor(x, 1);
+    return x;
+}
 
-// collects 8 tokens of a channel pair (one packed pair per token) into two rows of a [channel][token] tile
-struct Gather8 {
-    uint32_t a[4], b[4];
+// collects N tokens of a channel pair (one packed pair per token) into two rows of a [channel][token] tile
+template <int N>
+struct Gather {
+    uint32_t a[N / 2], b[N / 2];
     __device__ __forceinline__ void add(int x, uint32_t pair) {
         if (x & 1) { a[x >> 1] |= pair << 16;   b[x >> 1] |= pair & 0xffff0000u; }
         else       { a[x >> 1] = pair & 0xffffu; b[x >> 1] = pair >> 16; }
     }
     __device__ __forceinline__ void put(uint16_t *tile, int ot) const {
-        *reinterpret_cast<uint2 *>(&tile[ot]) = make_uint2(a[0], a[1]);
-        *reinterpret_cast<uint2 *>(&tile[ot + 4]) = make_uint2(a[2], a[3]);
-        *reinterpret_cast<uint2 *>(&tile[ot + LD]) = make_uint2(b[0], b[1]);
-        *reinterpret_cast<uint2 *>(&tile[ot + LD + 4]) = make_uint2(b[2], b[3]);
+#pragma unroll
+        for (int i = 0; i < N / 4; i++) {
+            *reinterpret_cast<uint2 *>(&tile[ot + 4 * i]) = make_uint2(a[2 * i], a[2 * i + 1]);
+            *reinterpret_cast<uint2 *>(&tile[ot + LD + 4 * i]) = make_uint2(b[2 * i], b[2 * i + 1]);
+        }
     }
-};
-
-struct FwdTiles {
-    uint16_t rd[SB * LD];    // r e^{excl-m}     [token][channel]  (bf16 head of the value)
-    uint16_t rdl[SB * LD];   //                                    (bf16 remainder)
-    uint16_t kd[SB * LD];    // k e^{m-incl}     [token][channel]
-    uint16_t kdl[SB * LD];
-    uint16_t rh[SB * LD];    // r e^{excl}       [token][channel]
-    uint16_t rhl[SB * LD];
-    uint16_t khT[SB * LD];   // k e^{b-incl}     [channel][token]
-    uint16_t khTl[SB * LD];
-    uint16_t vT[SB * LD];    // v                [channel][token]
-    float dec[4][HEAD];      // e^{b} per block and channel
-    float rho[SB];           // r . (u o k) per token
 };
 
 // One segment's summary for the time-parallel split: what the segment does to a
@@ -130,8 +161,21 @@ struct FwdTiles {
 // handed back (backward).  [key][value] fp32 plus one decay per key.
 constexpr int PART = HEAD * HEAD + HEAD;
 
+// ------------------------------------------------------------------- forward --
+struct FwdTiles {
+    uint16_t rh[SB * LD];    // r e^{excl}       [token][key]   bf16 head of the value
+    uint16_t rhl[SB * LD];   //                                 bf16 remainder
+    uint16_t kn[SB * LD];    // k e^{-incl}      [token][key]
+    uint16_t knl[SB * LD];
+    uint16_t khT[SB * LD];   // k e^{b-incl}     [key][token]
+    uint16_t khTl[SB * LD];
+    uint16_t vT[SB * LD];    // v                [value][token]
+    float dec[4][HEAD];      // e^{b} per block and key
+    float rho[SB];           // r . (u o k) per token
+};
+
 // Forward over one segment (`sps` 64-token steps) of one (batch, head); grid =
-// B*H*nseg.  The sequence is cut into nseg segments that run in parallel:
+// B*H*nseg, 4 wavefronts; wavefront w owns value columns 16w..16w+15 of the state.
 //   STATE_ONLY pass  (segments 0..nseg-2): from a zero state, leaves the segment's
 //                    summary in `part`;
 //   main pass        (all segments): folds the summaries of the earlier segments
@@ -139,7 +183,7 @@ constexpr int PART = HEAD * HEAD + HEAD;
 // ckpt (optional) receives the state at the start of every 64-token step,
 // [bh][step][key][value] fp32; the last segment writes s_out.
 template <bool PER_TOKEN_W, bool STATE_ONLY>
-__global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, int sps,
+__global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg, int sps,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
         bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, float *__restrict__ part,
@@ -167,7 +211,7 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
             for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
-        for (int gg = 0; gg < seg; gg++) {           // states of the earlier segments, in order
+        for (int gg = 0; gg < seg; gg++) {           // effect of the earlier segments, in order
             const float *pp = part + ((size_t)bh * nseg + gg) * PART;
 #pragma unroll
             for (int kk = 0; kk < 4; kk++)
@@ -195,7 +239,7 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
             const int t = sb * SB + 16 * wv + 8 * half + x;
             if (t < Tlen) {
                 const size_t o = base + (size_t)t * C + c0;
-                pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
+                if (!STATE_ONLY) pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
                 pk[x] = *reinterpret_cast<const uint32_t *>(k + o);
                 pv[x] = *reinterpret_cast<const uint32_t *>(v + o);
                 pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
@@ -207,7 +251,9 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
     };
 
     fetch(sb0);
+    PT_DECL
     for (int sb = sb0; sb < sb1; sb++) {
+        PT_MARK(4)
         // ---------------- prepare the scaled operands of 64 tokens
         {
             float ia[8], ib[8], la[8], lb[8];
@@ -223,31 +269,28 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
             const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
             const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
             const float tota = ra + oa, totb = rb + ob;
-            const float mida = half ? oa : ra, midb = half ? ob : rb;       // running sum after 8 tokens
-            const float ea_nm = __expf(-mida), eb_nm = __expf(-midb);
-            const float ea_mb = __expf(mida - tota), eb_mb = __expf(midb - totb);
+            const float enta = __expf(-tota), entb = __expf(-totb);
             float p[8];
-            Gather8 gk_h, gk_l, gv_;
+            Gather<8> gk_h, gk_l, gv_;
 #pragma unroll
             for (int x = 0; x < 8; x++) {
                 const float inca = ia[x] + offa, incb = ib[x] + offb;
-                const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]), kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
-                const float rha = rfa * __expf(inca - la[x]), rhb = rfb * __expf(incb - lb[x]);
+                const float kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
                 const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
                 const int o = (16 * wv + 8 * half + x) * LD + c0;
                 uint32_t hi, lo;
                 if (!STATE_ONLY) {
-                    split2(rha, rhb, hi, lo);
+                    const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]);
+                    split2(rfa * __expf(inca - la[x]), rfb * __expf(incb - lb[x]), hi, lo);
                     *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
                     *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
-                    split2(rha * ea_nm, rhb * eb_nm, hi, lo);
-                    *reinterpret_cast<uint32_t *>(&sm.rd[o]) = hi;
-                    *reinterpret_cast<uint32_t *>(&sm.rdl[o]) = lo;
-                    split2(kha * ea_mb, khb * eb_mb, hi, lo);
-                    *reinterpret_cast<uint32_t *>(&sm.kd[o]) = hi;
-                    *reinterpret_cast<uint32_t *>(&sm.kdl[o]) = lo;
+                    // k e^{-incl}; the block's last token has no later token and is never used
+                    const bool last = half && x == 7;
+                    split2(last ? 0.f : kha * enta, last ? 0.f : khb * entb, hi, lo);
+                    *reinterpret_cast<uint32_t *>(&sm.kn[o]) = hi;
+                    *reinterpret_cast<uint32_t *>(&sm.knl[o]) = lo;
+                    p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
                 }
-                p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
                 split2(kha, khb, hi, lo);
                 gk_h.add(x, hi);
                 gk_l.add(x, lo);
@@ -263,7 +306,9 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
                 if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
             }
         }
+        PT_MARK(0)
         __syncthreads();
+        PT_MARK(1)
         if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
 
         // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
@@ -277,46 +322,46 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             if (sb * SB + 16 * q >= Tlen) break;
+            const int row = 16 * q + n;
             const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
             if (!STATE_ONLY) {
-            // A^T[s][t] = sum_i kd[s][i] rd[t][i]; lane gets s = 4g+e, t = n
-            // (operands carried as bf16 head + remainder; head*head + rem*head + head*rem)
-            f4 at = {0.f, 0.f, 0.f, 0.f};
+                // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n.  Three
+                // independent accumulators (head*head, rem*head, head*rem) shorten the chain.
+                f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
+                // inter-block part of y: rh S, with S as head + remainder
+                f4 y0 = a0, y1 = a0, y2 = a0;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                const int row = 16 * q + n, c0 = 16 * kk + 4 * g, c1 = c0 + 16;
-                const s4 kh0 = frag(sm.kd, row, c0), kh1 = frag(sm.kd, row, c1);
-                const s4 rh0 = frag(sm.rd, row, c0), rh1 = frag(sm.rd, row, c1);
-                at = mma2(kh0, kh1, rh0, rh1, at);
-                at = mma2(frag(sm.kdl, row, c0), frag(sm.kdl, row, c1), rh0, rh1, at);
-                at = mma2(kh0, kh1, frag(sm.rdl, row, c0), frag(sm.rdl, row, c1), at);
-            }
-            const float rho_t = sm.rho[16 * q + n];
+                for (int kk = 0; kk < 4; kk += 2) {
+                    const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                    const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
+                    const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                    const s4 r0l = frag(sm.rhl, row, ca), r1l = frag(sm.rhl, row, cb);
+                    a0 = mma2(k0, k1, r0, r1, a0);
+                    a1 = mma2(frag(sm.knl, row, ca), frag(sm.knl, row, cb), r0, r1, a1);
+                    a2 = mma2(k0, k1, r0l, r1l, a2);
+                    s4 s0h, s0l, s1h, s1l;
+                    split4(S[kk], s0h, s0l);
+                    split4(S[kk + 1], s1h, s1l);
+                    y0 = mma2(r0, r1, s0h, s1h, y0);
+                    y1 = mma2(r0, r1, s0l, s1l, y1);
+                    y2 = mma2(r0l, r1l, s0h, s1h, y2);
+                }
+                f4 at = a0 + (a1 + a2);
+                const float rho_t = sm.rho[16 * q + n];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int s = 4 * g + e;
-                at[e] = s < n ? at[e] : (s == n ? rho_t : 0.f);
-            }
-            s4 a_hi, a_lo;                                  // A[t = n][s = 4g..4g+3]
-            split4(at, a_hi, a_lo);
-            f4 yt = {0.f, 0.f, 0.f, 0.f};
-            yt = mma2(a_hi, a_lo, v_op, v_op, yt);
+                for (int e = 0; e < 4; e++) {
+                    const int s = 4 * g + e;
+                    at[e] = s < n ? at[e] : (s == n ? rho_t : 0.f);
+                }
+                s4 a_hi, a_lo;                                  // A[t = n][s = 4g..4g+3]
+                split4(at, a_hi, a_lo);
+                f4 yt = y0 + (y1 + y2);
+                yt = mma2(a_hi, a_lo, v_op, v_op, yt);
 #pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                s4 s0h, s0l, s1h, s1l;
-                split4(S[kk], s0h, s0l);
-                split4(S[kk + 1], s1h, s1l);
-                const int row = 16 * q + n, ca = 16 * kk + 4 * g, cb = ca + 16;
-                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                yt = mma2(r0, r1, s0h, s1h, yt);
-                yt = mma2(r0, r1, s0l, s1l, yt);
-                yt = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, yt);
-            }
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int t = sb * SB + 16 * q + 4 * g + e;
-                if (y && t < Tlen) y[base + (size_t)t * C + 16 * wv + n] = bf16{bf16_bits(yt[e])};
-            }
+                for (int e = 0; e < 4; e++) {
+                    const int t = sb * SB + 16 * q + 4 * g + e;
+                    if (y && t < Tlen) y[base + (size_t)t * C + 16 * wv + n] = bf16{bf16_bits(yt[e])};
+                }
             }
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) {
@@ -327,8 +372,11 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
                              v_op, v_op, S[kk]);
             }
         }
+        PT_MARK(2)
         __syncthreads();
+        PT_MARK(3)
     }
+    PT_PRINT(STATE_ONLY ? "fwd-state" : "fwd")
     if (STATE_ONLY) {
         float *pp = part + ((size_t)bh * nseg + seg) * PART;
 #pragma unroll
@@ -348,12 +396,11 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
     }
 }
 
-
 // ------------------------------------------------------------------ backward --
-// Walks the 64-token steps from the last to the first.  Per step: prepare the
-// operands, rebuild the state at the start of each of its four blocks from the
-// step's checkpoint, then take the blocks in reverse.  With G the gradient of
-// the state at a block's end, P[t][s] = gy_t . v_s, rh = r e^{excl}, kh = k e^{b-incl}:
+// Walks the 64-token steps of a segment from the last to the first.  Per step:
+// prepare the operands, rebuild the state at the start of each of its four blocks
+// from the step's checkpoint, then take the blocks in reverse.  With G the gradient
+// of the state at a block's end, P[t][s] = gy_t . v_s, rh = r e^{excl}, kh = k e^{b-incl}:
 //
 //   gr_t = e^{excl_t} (gy_t S^T) + e^{excl_t-b} sum_{s<t} P[t][s] kh_s + u k_t P[t][t]
 //   gk_s = e^{-incl_s} sum_{t>s} P[t][s] rh_t + e^{b-incl_s} (v_s G^T) + u r_s P[s][s]
@@ -362,16 +409,20 @@ __global__ __launch_bounds__(NT) void forward(int Tlen, int C, int H, int nseg, 
 //
 // and the decay gradient from the running sum  A_{t-1} = A_t + r_t gr_t - k_t gk_t,
 // dL/dlog w_t = A_t - k_t (gk_t - u r_t P[t][t]),  re-anchored at every step end
-// to sum_j G o S.  Each wavefront owns key channels 16w..16w+15 for gr, gk, gw
-// (state and G held value-major for that slice) and value channels 16w..16w+15
-// for gv (a second copy of G, key-major), so no result crosses wavefronts.
+// to sum_j G o S.
+//
+// Eight wavefronts: all of them prepare the operands; then wavefronts 0-3 ("key
+// side", key channels 16w..16w+15) rebuild the state and produce gr, gk, gw, gu with
+// G held value-major, while wavefronts 4-7 ("value side", value channels 16w..16w+15)
+// produce gv with a second, key-major copy of G.  Neither side needs anything the
+// other computes, so two wavefronts per SIMD hide each other's latencies.
 struct BwdTiles {
     uint16_t gy[SB * LD];    // gy              [token][value]
     uint16_t v[SB * LD];     // v               [token][value]
-    uint16_t rd[SB * LD];    // r e^{excl-m}    [token][key]   head / remainder
-    uint16_t rdl[SB * LD];
-    uint16_t kd[SB * LD];    // k e^{m-incl}    [token][key]
-    uint16_t kdl[SB * LD];
+    uint16_t rh[SB * LD];    // r e^{excl}      [token][key]   head / remainder
+    uint16_t rhl[SB * LD];
+    uint16_t kn[SB * LD];    // k e^{-incl}     [token][key]
+    uint16_t knl[SB * LD];
     uint16_t kh[SB * LD];    // k e^{b-incl}    [token][key]
     uint16_t khl[SB * LD];
     uint16_t gyT[SB * LD];   // gy              [value][token]
@@ -384,17 +435,11 @@ struct BwdTiles {
     float lw[SB * HEAD];     // log w                                         [token][key]
     float tot[4][HEAD];      // b per block and key
     float dec[4][HEAD];      // e^{b}
-    float rho[SB];
+    float rho[2][SB];        // r . (u o k) per token, one partial sum per half of the channels
 };
 
-__device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane groups of 16
-    x += __shfl_xor(x, 16);
-    x += __shfl_xor(x, 32);
-    return x;
-}
-
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H, int nseg, int sps,
+__global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nseg, int sps,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
         const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
@@ -404,25 +449,28 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H, int nseg,
     extern __shared__ __align__(16) unsigned char smem_raw[];
     BwdTiles &sm = *reinterpret_cast<BwdTiles *>(smem_raw);
     const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
-    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const int tid = threadIdx.x, w8 = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const bool key_side = w8 < 4;
+    const int wv = w8 & 3;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
     const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
-    const int own = 16 * wv + n;                 // key channel (gr, gk, gw) / value channel (gv) of this lane
+    const int own = 16 * wv + n;                 // key channel (key side) / value channel (value side) of this lane
     const float u_i = u[h * HEAD + own];
 
-    // GT[kk][e] = G[key own][value 16kk+4g+e];  GJ[kk][e] = G[key 16kk+4g+e][value own]
-    f4 GT[4], GJ[4];
+    // key side:   G[kk][e] = G[key own][value 16kk+4g+e]
+    // value side: G[kk][e] = G[key 16kk+4g+e][value own]
+    f4 G[4];
     {
         const float *gp = gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                GT[kk][e] = gp ? gp[own * HEAD + 16 * kk + 4 * g + e] : 0.f;
-                GJ[kk][e] = gp ? gp[(16 * kk + 4 * g + e) * HEAD + own] : 0.f;
+                const int x = 16 * kk + 4 * g + e;
+                G[kk][e] = gp ? (key_side ? gp[own * HEAD + x] : gp[x * HEAD + own]) : 0.f;
             }
-        for (int gg = nseg - 1; gg > seg; gg--) {      // gradients through the later segments, last first
+        for (int gg = nseg - 1; gg > seg; gg--) {      // effect of the later segments, last first
             const float *pp = gpart + ((size_t)bh * nseg + gg) * PART;
             const float d_own = pp[HEAD * HEAD + own];
 #pragma unroll
@@ -430,27 +478,29 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H, int nseg,
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int x = 16 * kk + 4 * g + e;
-                    GT[kk][e] = fmaf(d_own, GT[kk][e], pp[own * HEAD + x]);
-                    GJ[kk][e] = fmaf(pp[HEAD * HEAD + x], GJ[kk][e], pp[x * HEAD + own]);
+                    G[kk][e] = key_side ? fmaf(d_own, G[kk][e], pp[own * HEAD + x])
+                                        : fmaf(pp[HEAD * HEAD + x], G[kk][e], pp[x * HEAD + own]);
                 }
         }
     }
     float A_run = 0.f, gu_acc = 0.f, gw_acc = 0.f;
 
-    // staging role (as in forward): block wv, tokens 8*half.., channels c0, c0+1
-    const int half = lane >> 5, c0 = 2 * (lane & 31);
+    // staging role: block sq of the step, tokens 8*half + 4*quarter .. +3 of it, channels c0, c0+1
+    const int sq = w8 >> 1, half = lane >> 5, quarter = (lane >> 4) & 1;
+    const int chh = w8 & 1, c0 = 2 * (16 * chh + (lane & 15));
+    const int tk0 = 16 * sq + 8 * half + 4 * quarter;
     const float2 u_c = *reinterpret_cast<const float2 *>(u + h * HEAD + c0);
     float2 l_const = make_float2(0.f, 0.f);
     if (!PER_TOKEN_W) {
         l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
         l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
     }
-    uint32_t pr[8], pk[8], pv[8], pg[8];
-    float2 pw[8];
+    uint32_t pr[4], pk[4], pv[4], pg[4];
+    float2 pw[4];
     auto fetch = [&](int sb) {
 #pragma unroll
-        for (int x = 0; x < 8; x++) {
-            const int t = sb * SB + 16 * wv + 8 * half + x;
+        for (int x = 0; x < 4; x++) {
+            const int t = sb * SB + tk0 + x;
             if (t < Tlen) {
                 const size_t o = base + (size_t)t * C + c0;
                 pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
@@ -466,267 +516,299 @@ __global__ __launch_bounds__(NT) void backward(int Tlen, int C, int H, int nseg,
     };
 
     fetch(sb1 - 1);
+    PT_DECL
     for (int sb = sb1 - 1; sb >= sb0; sb--) {
-        // ---------------- prepare the operands of 64 tokens
+        PT_MARK(4)
+        // ---------------- prepare the operands of 64 tokens (all 8 wavefronts)
         {
-            float ia[8], ib[8], la[8], lb[8];
+            float ia[4], ib[4], la[4], lb[4];
             float ra = 0.f, rb = 0.f;
 #pragma unroll
-            for (int x = 0; x < 8; x++) {
+            for (int x = 0; x < 4; x++) {
                 la[x] = PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
                 lb[x] = PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
                 ra += la[x]; rb += lb[x];
                 ia[x] = ra; ib[x] = rb;
             }
-            const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
-            const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
-            const float tota = ra + oa, totb = rb + ob;
-            const float mida = half ? oa : ra, midb = half ? ob : rb;
-            const float ea_nm = __expf(-mida), eb_nm = __expf(-midb);
-            const float ea_mb = __expf(mida - tota), eb_mb = __expf(midb - totb);
-            float p[8];
-            Gather8 gk_h, gk_l, gr_h, gr_l, gv_, gg_;
+            // the block's four quarters sit in lanes ^16 and ^32
+            const float qa = __shfl_xor(ra, 16), qb = __shfl_xor(rb, 16);
+            const float pa = ra + qa, pb = rb + qb;                  // this half's 8 tokens
+            const float ha = __shfl_xor(pa, 32), hb = __shfl_xor(pb, 32);
+            const float tota = pa + ha, totb = pb + hb;
+            const float offa = (quarter ? qa : 0.f) + (half ? ha : 0.f), offb = (quarter ? qb : 0.f) + (half ? hb : 0.f);
+            const float enta = __expf(-tota), entb = __expf(-totb);
+            float p[4];
+            Gather<4> gk_h, gk_l, gr_h, gr_l, gv_, gg_;
 #pragma unroll
-            for (int x = 0; x < 8; x++) {
+            for (int x = 0; x < 4; x++) {
                 const float inca = ia[x] + offa, incb = ib[x] + offb;
                 const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]), kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
-                const float rha = rfa * __expf(inca - la[x]), rhb = rfb * __expf(incb - lb[x]);
                 const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
-                const int tk = 16 * wv + 8 * half + x;
+                const int tk = tk0 + x;
                 const int o = tk * LD + c0;
                 uint32_t hi, lo;
                 *reinterpret_cast<uint32_t *>(&sm.gy[o]) = pg[x];
                 *reinterpret_cast<uint32_t *>(&sm.v[o]) = pv[x];
-                split2(rha * ea_nm, rhb * eb_nm, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.rd[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.rdl[o]) = lo;
-                split2(kha * ea_mb, khb * eb_mb, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.kd[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.kdl[o]) = lo;
+                split2(rfa * __expf(inca - la[x]), rfb * __expf(incb - lb[x]), hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
+                gr_h.add(x, hi);
+                gr_l.add(x, lo);
+                const bool last = half && quarter && x == 3;       // no later token in the block: never used
+                split2(last ? 0.f : kha * enta, last ? 0.f : khb * entb, hi, lo);
+                *reinterpret_cast<uint32_t *>(&sm.kn[o]) = hi;
+                *reinterpret_cast<uint32_t *>(&sm.knl[o]) = lo;
                 split2(kha, khb, hi, lo);
                 *reinterpret_cast<uint32_t *>(&sm.kh[o]) = hi;
                 *reinterpret_cast<uint32_t *>(&sm.khl[o]) = lo;
                 gk_h.add(x, hi);
                 gk_l.add(x, lo);
-                split2(rha, rhb, hi, lo);
-                gr_h.add(x, hi);
-                gr_l.add(x, lo);
                 gv_.add(x, pv[x]);
                 gg_.add(x, pg[x]);
                 *reinterpret_cast<float2 *>(&sm.incl[tk * HEAD + c0]) = make_float2(inca, incb);
                 *reinterpret_cast<float2 *>(&sm.lw[tk * HEAD + c0]) = make_float2(la[x], lb[x]);
                 p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
             }
-            const int ot = c0 * LD + 16 * wv + 8 * half;
+            const int ot = c0 * LD + tk0;
             gk_h.put(sm.khT, ot);
             gk_l.put(sm.khTl, ot);
             gr_h.put(sm.rhT, ot);
             gr_l.put(sm.rhTl, ot);
             gv_.put(sm.vT, ot);
             gg_.put(sm.gyT, ot);
-            if (!half) {
-                *reinterpret_cast<float2 *>(&sm.tot[wv][c0]) = make_float2(tota, totb);
-                *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(tota), __expf(totb));
+            if (!half && !quarter) {
+                *reinterpret_cast<float2 *>(&sm.tot[sq][c0]) = make_float2(tota, totb);
+                *reinterpret_cast<float2 *>(&sm.dec[sq][c0]) = make_float2(__expf(tota), __expf(totb));
             }
-            const float tot_p = sum8_over_half(p, lane);
-            if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
+            const float tot_p = sum4_over_16(p, lane);
+            if ((lane & 3) == 0) sm.rho[chh][tk0 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1)] = tot_p;
         }
+        PT_MARK(0)
         __syncthreads();
+        PT_MARK(1)
         if (sb > sb0) fetch(sb - 1);
 
-        // ---------------- rebuild the state at the start of each block (value-major slice: key `own`)
-        f4 ST[4];
-        {
-            const float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD + own * HEAD;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                const float4 x = *reinterpret_cast<const float4 *>(cp + 16 * kk + 4 * g);
-                ST[kk][0] = x.x; ST[kk][1] = x.y; ST[kk][2] = x.z; ST[kk][3] = x.w;
-            }
-        }
-        s4 Sh[4][4], Sl[4][4];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) split4(ST[kk], Sh[q][kk], Sl[q][kk]);
-            if (sb * SB + 16 * q >= Tlen) continue;
-            const float dq = sm.dec[q][own];
-            const s4 khf = frag(sm.khT, own, 16 * q + 4 * g), khfl = frag(sm.khTl, own, 16 * q + 4 * g);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                ST[kk] = ST[kk] * dq;
-                const s4 vf_ = frag(sm.vT, 16 * kk + n, 16 * q + 4 * g);
-                ST[kk] = mma2(vf_, vf_, khf, khfl, ST[kk]);
-            }
-        }
-        {   // anchor of the decay-gradient sum at the end of this step: sum_j G o S
-            float a = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) a = fmaf(GT[kk][e], ST[kk][e], a);
-            A_run = group_sum4(a);
-        }
-
-        // ---------------- the four blocks, last first
-#pragma unroll
-        for (int q = 3; q >= 0; q--) {
-            if (sb * SB + 16 * q >= Tlen) continue;
-            const int row = 16 * q + n;
-            s4 gyf[4], vf[4];
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                gyf[kk] = frag(sm.gy, row, 16 * kk + 4 * g);
-                vf[kk] = frag(sm.v, row, 16 * kk + 4 * g);
-            }
-            // pt[e] = P[t = 4g+e][s = n],  ptT[e] = P[t = n][s = 4g+e]
-            f4 pt = {0.f, 0.f, 0.f, 0.f}, ptT = {0.f, 0.f, 0.f, 0.f};
-            pt = mma2(gyf[0], gyf[1], vf[0], vf[1], pt);
-            pt = mma2(gyf[2], gyf[3], vf[2], vf[3], pt);
-            ptT = mma2(vf[0], vf[1], gyf[0], gyf[1], ptT);
-            ptT = mma2(vf[2], vf[3], gyf[2], gyf[3], ptT);
-            float pd[4];                                   // P[t][t] for this lane's tokens t = 4g+e
-            f4 pm, pTm;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                pd[e] = __shfl(pt[e], (lane & 48) | (4 * g + e));
-                pm[e] = (4 * g + e > n) ? pt[e] : 0.f;     // later tokens t > s
-                pTm[e] = (4 * g + e < n) ? ptT[e] : 0.f;   // earlier tokens s < t
-            }
-            s4 pm_h, pm_l, pT_h, pT_l;
-            split4(pm, pm_h, pm_l);
-            split4(pTm, pT_h, pT_l);
-
-            // the forward's masked matrix: at[e] = A~[t = 4g+e][s = n]
-            f4 at = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                const s4 rh0 = frag(sm.rd, row, ca), rh1 = frag(sm.rd, row, cb);
-                const s4 kh0 = frag(sm.kd, row, ca), kh1 = frag(sm.kd, row, cb);
-                at = mma2(rh0, rh1, kh0, kh1, at);
-                at = mma2(frag(sm.rdl, row, ca), frag(sm.rdl, row, cb), kh0, kh1, at);
-                at = mma2(rh0, rh1, frag(sm.kdl, row, ca), frag(sm.kdl, row, cb), at);
-            }
+        if (key_side) {
+            // ---------------- rebuild the state at the start of each block: ST[kk][e] = S[key own][value 16kk+4g+e]
+            f4 ST[4];
             {
-                const float rho_s = sm.rho[16 * q + n];
-#pragma unroll
-                for (int e = 0; e < 4; e++) at[e] = (4 * g + e > n) ? at[e] : ((4 * g + e == n) ? rho_s : 0.f);
-            }
-            s4 a_h, a_l;
-            split4(at, a_h, a_l);
-
-            const s4 gyTf = frag(sm.gyT, own, 16 * q + 4 * g);     // gy[t = 4g..][value own]
-            const s4 khTf = frag(sm.khT, own, 16 * q + 4 * g);     // kh[s = 4g..][key own]
-            const s4 khTfl = frag(sm.khTl, own, 16 * q + 4 * g);
-            const s4 rhTf = frag(sm.rhT, own, 16 * q + 4 * g);     // rh[t = 4g..][key own]
-            const s4 rhTfl = frag(sm.rhTl, own, 16 * q + 4 * g);
-
-            // gv[s = 4g+e][value own]
-            f4 gvt = {0.f, 0.f, 0.f, 0.f};
-            gvt = mma2(a_h, a_l, gyTf, gyTf, gvt);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                s4 g0h, g0l, g1h, g1l;
-                split4(GJ[kk], g0h, g0l);
-                split4(GJ[kk + 1], g1h, g1l);
-                const s4 k0 = frag(sm.kh, row, 16 * kk + 4 * g), k1 = frag(sm.kh, row, 16 * kk + 16 + 4 * g);
-                gvt = mma2(k0, k1, g0h, g1h, gvt);
-                gvt = mma2(k0, k1, g0l, g1l, gvt);
-                gvt = mma2(frag(sm.khl, row, 16 * kk + 4 * g), frag(sm.khl, row, 16 * kk + 16 + 4 * g), g0h, g1h, gvt);
-            }
-            // gr, gk pieces at [token 4g+e][key own]
-            f4 q1 = {0.f, 0.f, 0.f, 0.f}, q2 = {0.f, 0.f, 0.f, 0.f}, q3 = {0.f, 0.f, 0.f, 0.f}, q4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                q1 = mma2(gyf[kk], gyf[kk + 1], Sh[q][kk], Sh[q][kk + 1], q1);
-                q1 = mma2(gyf[kk], gyf[kk + 1], Sl[q][kk], Sl[q][kk + 1], q1);
-                s4 g0h, g0l, g1h, g1l;
-                split4(GT[kk], g0h, g0l);
-                split4(GT[kk + 1], g1h, g1l);
-                q4 = mma2(vf[kk], vf[kk + 1], g0h, g1h, q4);
-                q4 = mma2(vf[kk], vf[kk + 1], g0l, g1l, q4);
-            }
-            q2 = mma2(pT_h, pT_l, khTf, khTf, q2);
-            q2 = mma(pT_h, khTfl, q2);
-            q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);
-            q3 = mma(pm_h, rhTfl, q3);
-
-            const float tot_i = sm.tot[q][own], mid_i = sm.incl[(16 * q + 7) * HEAD + own];
-            float c[4], z[4], lfac[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int tk = 16 * q + 4 * g + e;
-                const int t = sb * SB + tk;
-                const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
-                // r, k back from their re-centred head + remainder (16 mantissa bits)
-                const float rr = (bf2f(sm.rd[tk * LD + own]) + bf2f(sm.rdl[tk * LD + own])) * __expf(mid_i - exc);
-                const float kr = (bf2f(sm.kd[tk * LD + own]) + bf2f(sm.kdl[tk * LD + own])) * __expf(inc - mid_i);
-                const float grv = __expf(exc) * q1[e] + __expf(exc - tot_i) * q2[e] + u_i * kr * pd[e];
-                const float gkn = __expf(-inc) * q3[e] + __expf(tot_i - inc) * q4[e];
-                const float gkv = gkn + u_i * rr * pd[e];
-                c[e] = rr * grv - kr * gkv;
-                z[e] = kr * gkn;
-                lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
-                gu_acc = fmaf(rr * kr, pd[e], gu_acc);
-                if (t < Tlen) {
-                    const size_t o = base + (size_t)t * C;
-                    gr[o + own] = bf16{bf16_bits(grv)};
-                    gk[o + own] = bf16{bf16_bits(gkv)};
-                    gv[o + own] = bf16{bf16_bits(gvt[e])};
-                }
-            }
-            {   // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over later tokens of c
-                const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
-                const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
-                const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
-                const float all = group_sum4(mine);
-                const float suf[4] = {suf0, suf1, suf2, 0.f};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float Dt = A_run + later + suf[e] - z[e];
-                    const int t = sb * SB + 16 * q + 4 * g + e;
-                    if (PER_TOKEN_W) {
-                        if (t < Tlen) gw_tok[base + (size_t)t * C + own] = Dt * lfac[e];
-                    } else {
-                        gw_acc += (t < Tlen) ? Dt : 0.f;
-                    }
-                }
-                A_run += all;
-            }
-            // G <- e^{b} o G + rh^T gy, both copies
-            {
-                const float dq = sm.dec[q][own];
+                const float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD + own * HEAD;
 #pragma unroll
                 for (int kk = 0; kk < 4; kk++) {
-                    GT[kk] = GT[kk] * dq;
-                    const s4 gT_ = frag(sm.gyT, 16 * kk + n, 16 * q + 4 * g);
-                    GT[kk] = mma2(gT_, gT_, rhTf, rhTfl, GT[kk]);
+                    const float4 x = *reinterpret_cast<const float4 *>(cp + 16 * kk + 4 * g);
+                    ST[kk][0] = x.x; ST[kk][1] = x.y; ST[kk][2] = x.z; ST[kk][3] = x.w;
+                }
+            }
+            f4 Q1[4];                        // gy S^T per block, taken while S passes by: Q1[q][e] at [token 4g+e][key own]
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                Q1[q] = f4{0.f, 0.f, 0.f, 0.f};
+                if (sb * SB + 16 * q >= Tlen) continue;
+                {
+                    s4 sh[4], sl[4];
+#pragma unroll
+                    for (int kk = 0; kk < 4; kk++) split4(ST[kk], sh[kk], sl[kk]);
+                    f4 qa = {0.f, 0.f, 0.f, 0.f}, qb = qa;
+#pragma unroll
+                    for (int kk = 0; kk < 4; kk += 2) {
+                        const s4 y0 = frag(sm.gy, 16 * q + n, 16 * kk + 4 * g), y1 = frag(sm.gy, 16 * q + n, 16 * kk + 16 + 4 * g);
+                        qa = mma2(y0, y1, sh[kk], sh[kk + 1], qa);
+                        qb = mma2(y0, y1, sl[kk], sl[kk + 1], qb);
+                    }
+                    Q1[q] = qa + qb;
+                }
+                const float dq = sm.dec[q][own];
+                const s4 khf = frag(sm.khT, own, 16 * q + 4 * g), khfl = frag(sm.khTl, own, 16 * q + 4 * g);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    ST[kk] = ST[kk] * dq;
+                    const s4 vf_ = frag(sm.vT, 16 * kk + n, 16 * q + 4 * g);
+                    ST[kk] = mma2(vf_, vf_, khf, khfl, ST[kk]);
+                }
+            }
+            {   // anchor of the decay-gradient sum at the end of this step: sum_j G o S
+                float a = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) a = fmaf(G[kk][e], ST[kk][e], a);
+                A_run = group_sum4(a);
+            }
+            PT_MARK(5)
+            // ---------------- the four blocks, last first: gr, gk, gw, gu
+#pragma unroll
+            for (int q = 3; q >= 0; q--) {
+                if (sb * SB + 16 * q >= Tlen) continue;
+                const int row = 16 * q + n;
+                s4 gyf[4], vf[4];
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    gyf[kk] = frag(sm.gy, row, 16 * kk + 4 * g);
+                    vf[kk] = frag(sm.v, row, 16 * kk + 4 * g);
+                }
+                // pt[e] = P[t = 4g+e][s = n],  ptT[e] = P[t = n][s = 4g+e]
+                f4 pt = {0.f, 0.f, 0.f, 0.f}, ptT = pt;
+                pt = mma2(gyf[0], gyf[1], vf[0], vf[1], pt);
+                ptT = mma2(vf[0], vf[1], gyf[0], gyf[1], ptT);
+                pt = mma2(gyf[2], gyf[3], vf[2], vf[3], pt);
+                ptT = mma2(vf[2], vf[3], gyf[2], gyf[3], ptT);
+                // state-gradient part while P is in flight: q4 = v G^T
+                f4 q1 = Q1[q], q4 = {0.f, 0.f, 0.f, 0.f}, q4b = q4;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk += 2) {
+                    s4 g0h, g0l, g1h, g1l;
+                    split4(G[kk], g0h, g0l);
+                    split4(G[kk + 1], g1h, g1l);
+                    q4 = mma2(vf[kk], vf[kk + 1], g0h, g1h, q4);
+                    q4b = mma2(vf[kk], vf[kk + 1], g0l, g1l, q4b);
+                }
+                float pd[4];                                   // P[t][t] for this lane's tokens t = 4g+e
+                f4 pm, pTm;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    pd[e] = __shfl(pt[e], (lane & 48) | (4 * g + e));
+                    pm[e] = (4 * g + e > n) ? pt[e] : 0.f;     // later tokens t > s
+                    pTm[e] = (4 * g + e < n) ? ptT[e] : 0.f;   // earlier tokens s < t
+                }
+                s4 pm_h, pm_l, pT_h, pT_l;
+                split4(pm, pm_h, pm_l);
+                split4(pTm, pT_h, pT_l);
+                const s4 khTf = frag(sm.khT, own, 16 * q + 4 * g);     // kh[s = 4g..][key own]
+                const s4 khTfl = frag(sm.khTl, own, 16 * q + 4 * g);
+                const s4 rhTf = frag(sm.rhT, own, 16 * q + 4 * g);     // rh[t = 4g..][key own]
+                const s4 rhTfl = frag(sm.rhTl, own, 16 * q + 4 * g);
+                f4 q2 = {0.f, 0.f, 0.f, 0.f}, q2b = q2, q3 = q2, q3b = q2;
+                q2 = mma2(pT_h, pT_l, khTf, khTf, q2);
+                q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);
+                q2b = mma(pT_h, khTfl, q2b);
+                q3b = mma(pm_h, rhTfl, q3b);
+                q4 += q4b; q2 += q2b; q3 += q3b;
+
+                const float tot_i = sm.tot[q][own], ent_i = __expf(-tot_i);
+                float c[4], z[4], lfac[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int tk = 16 * q + 4 * g + e;
+                    const int t = sb * SB + tk;
+                    const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
+                    const float E1 = __expf(exc), E2 = __expf(tot_i - inc);
+                    // r, k back from their scaled head + remainder (16 mantissa bits)
+                    const float rr = (bf2f(sm.rh[tk * LD + own]) + bf2f(sm.rhl[tk * LD + own])) * __expf(-exc);
+                    const float kr = (bf2f(sm.kh[tk * LD + own]) + bf2f(sm.khl[tk * LD + own])) * __expf(inc - tot_i);
+                    const float grv = E1 * (q1[e] + ent_i * q2[e]) + u_i * kr * pd[e];
+                    const float gkn = E2 * (ent_i * q3[e] + q4[e]);
+                    const float gkv = gkn + u_i * rr * pd[e];
+                    c[e] = rr * grv - kr * gkv;
+                    z[e] = kr * gkn;
+                    lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
+                    gu_acc = fmaf(rr * kr, pd[e], gu_acc);
+                    if (t < Tlen) {
+                        const size_t o = base + (size_t)t * C;
+                        gr[o + own] = bf16{bf16_bits(grv)};
+                        gk[o + own] = bf16{bf16_bits(gkv)};
+                    }
+                }
+                {   // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over later tokens of c
+                    const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
+                    const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
+                    const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
+                    const float all = group_sum4(mine);
+                    const float suf[4] = {suf0, suf1, suf2, 0.f};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float Dt = A_run + later + suf[e] - z[e];
+                        const int t = sb * SB + 16 * q + 4 * g + e;
+                        if (PER_TOKEN_W) {
+                            if (t < Tlen) gw_tok[base + (size_t)t * C + own] = Dt * lfac[e];
+                        } else {
+                            gw_acc += (t < Tlen) ? Dt : 0.f;
+                        }
+                    }
+                    A_run += all;
+                }
+                {   // G <- e^{b} o G + rh^T gy  (value-major copy: one decay per lane)
+                    const float dq = sm.dec[q][own];
+#pragma unroll
+                    for (int kk = 0; kk < 4; kk++) {
+                        G[kk] = G[kk] * dq;
+                        const s4 gT_ = frag(sm.gyT, 16 * kk + n, 16 * q + 4 * g);
+                        G[kk] = mma2(gT_, gT_, rhTf, rhTfl, G[kk]);
+                    }
+                }
+            }
+        } else {
+            // ---------------- value side: gv for value channel `own`, key-major G
+#pragma unroll
+            for (int q = 3; q >= 0; q--) {
+                if (sb * SB + 16 * q >= Tlen) continue;
+                const int row = 16 * q + n;
+                // the forward's masked matrix: at[e] = A~[t = 4g+e][s = n], three independent accumulators;
+                // and kh G with G as head + remainder
+                f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, g0 = a0, g1 = a0, g2 = a0;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk += 2) {
+                    const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                    const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                    const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
+                    a0 = mma2(r0, r1, k0, k1, a0);
+                    a1 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), k0, k1, a1);
+                    a2 = mma2(r0, r1, frag(sm.knl, row, ca), frag(sm.knl, row, cb), a2);
+                    s4 g0h, g0l, g1h, g1l;
+                    split4(G[kk], g0h, g0l);
+                    split4(G[kk + 1], g1h, g1l);
+                    const s4 h0 = frag(sm.kh, row, ca), h1 = frag(sm.kh, row, cb);
+                    g0 = mma2(h0, h1, g0h, g1h, g0);
+                    g1 = mma2(h0, h1, g0l, g1l, g1);
+                    g2 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g2);
+                }
+                f4 at = a0 + (a1 + a2);
+                {
+                    const float rho_s = sm.rho[0][16 * q + n] + sm.rho[1][16 * q + n];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) at[e] = (4 * g + e > n) ? at[e] : ((4 * g + e == n) ? rho_s : 0.f);
+                }
+                s4 a_h, a_l;
+                split4(at, a_h, a_l);
+                const s4 gyTf = frag(sm.gyT, own, 16 * q + 4 * g);     // gy[t = 4g..][value own]
+                f4 gvt = g0 + (g1 + g2);
+                gvt = mma2(a_h, a_l, gyTf, gyTf, gvt);                 // gv[s = 4g+e][value own]
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int t = sb * SB + 16 * q + 4 * g + e;
+                    if (t < Tlen) gv[base + (size_t)t * C + own] = bf16{bf16_bits(gvt[e])};
+                }
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {   // G <- e^{b} o G + rh^T gy  (key-major copy: one decay per row)
                     const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
-                    GJ[kk][0] *= d4.x; GJ[kk][1] *= d4.y; GJ[kk][2] *= d4.z; GJ[kk][3] *= d4.w;
-                    GJ[kk] = mma2(frag(sm.rhT, 16 * kk + n, 16 * q + 4 * g), frag(sm.rhTl, 16 * kk + n, 16 * q + 4 * g),
-                                  gyTf, gyTf, GJ[kk]);
+                    G[kk][0] *= d4.x; G[kk][1] *= d4.y; G[kk][2] *= d4.z; G[kk][3] *= d4.w;
+                    G[kk] = mma2(frag(sm.rhT, 16 * kk + n, 16 * q + 4 * g), frag(sm.rhTl, 16 * kk + n, 16 * q + 4 * g),
+                                 gyTf, gyTf, G[kk]);
                 }
             }
         }
+        PT_MARK(2)
         __syncthreads();
+        PT_MARK(3)
     }
+    PT_PRINT("bwd")
 
-    if (gs_in && seg == 0) {
-        float *gp = gs_in + (size_t)bh * HEAD * HEAD + own * HEAD;
+    if (key_side) {
+        if (gs_in && seg == 0) {
+            float *gp = gs_in + (size_t)bh * HEAD * HEAD + own * HEAD;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++)
-            *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(GT[kk][0], GT[kk][1], GT[kk][2], GT[kk][3]);
-    }
-    gu_acc = group_sum4(gu_acc);
-    gw_acc = group_sum4(gw_acc);
-    if (g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
-        const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
-        gu_part[po] = gu_acc;
-        if (!PER_TOKEN_W) {
-            bool fl;
-            const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
-            gw_part[po] = fl ? 0.f : gw_acc * l;
+            for (int kk = 0; kk < 4; kk++)
+                *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(G[kk][0], G[kk][1], G[kk][2], G[kk][3]);
+        }
+        gu_acc = group_sum4(gu_acc);
+        gw_acc = group_sum4(gw_acc);
+        if (g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
+            const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
+            gu_part[po] = gu_acc;
+            if (!PER_TOKEN_W) {
+                bool fl;
+                const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
+                gw_part[po] = fl ? 0.f : gw_acc * l;
+            }
         }
     }
 }
@@ -744,7 +826,7 @@ struct GPassTiles {
 };
 
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT) void gradient_pass(int Tlen, int C, int H, int nseg, int sps,
+__global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, int nseg, int sps,
         const bf16 *__restrict__ r, const float *__restrict__ wraw, const bf16 *__restrict__ gy,
         float *__restrict__ gpart, int floor_decay)
 {
@@ -796,7 +878,7 @@ __global__ __launch_bounds__(NT) void gradient_pass(int Tlen, int C, int H, int 
             }
             const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
             const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
-            Gather8 gr_h, gr_l, gg_;
+            Gather<8> gr_h, gr_l, gg_;
 #pragma unroll
             for (int x = 0; x < 8; x++) {
                 uint32_t hi, lo;
@@ -839,15 +921,16 @@ __global__ __launch_bounds__(NT) void gradient_pass(int Tlen, int C, int H, int 
         }
 }
 
+// ------------------------------------------------------------------ launchers --
 size_t checkpoint_bytes(int B, int Tlen, int H) {
     return (size_t)B * H * ((Tlen + SB - 1) / SB) * HEAD * HEAD * sizeof(float);
 }
 
 // How many time segments run in parallel for one (batch, head): enough workgroups
 // to give every CU about two, each segment at least four 64-token steps long.
-// RWKV_WKV_NSEG overrides it (tuning aid).
+// wkv_tune(WKV_TUNE_SEGMENTS) / RWKV_WKV_NSEG override it.
 struct SegPlan { int nseg, sps; };
-inline int &forced_segments() {          // 0 = choose automatically (wkv_tune)
+inline int &forced_segments() {          // 0 = choose automatically
     static int v = [] { const char *e = getenv("RWKV_WKV_NSEG"); return e ? atoi(e) : 0; }();
     return v;
 }
@@ -892,7 +975,7 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
     float *ckpt = (workspace && keep_ckpt) ? (float *)workspace : nullptr;
     float *part = workspace ? (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H)) : nullptr;
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v;
-    dim3 block(NT);
+    dim3 block(NT_F);
     if (pl.nseg > 1) {
         dim3 grid(B * H * (pl.nseg - 1));
         if (per_token)
@@ -939,9 +1022,8 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
     SegPlan pl = plan_segments(B * H, Tlen);
     if (pl.nseg > MAX_SEG) pl = SegPlan{1, (Tlen + SB - 1) / SB};
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v, *gg = (const bf16 *)gy;
-    dim3 block(NT);
     if (pl.nseg > 1) {
-        dim3 grid(B * H * (pl.nseg - 1));
+        dim3 grid(B * H * (pl.nseg - 1)), block(NT_F);
         if (per_token)
             hipLaunchKernelGGL((gradient_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, rr, w, gg, gpart,
                                floor_decay);
@@ -951,7 +1033,7 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(B * H * pl.nseg);
+    dim3 grid(B * H * pl.nseg), block(NT_B);
     prof_begin(KID_CHUNK_BACKWARD, s);
     if (per_token)
         hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv, w,
