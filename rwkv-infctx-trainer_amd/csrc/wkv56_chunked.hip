@@ -926,9 +926,11 @@ size_t checkpoint_bytes(int B, int Tlen, int H) {
     return (size_t)B * H * ((Tlen + SB - 1) / SB) * HEAD * HEAD * sizeof(float);
 }
 
-// How many time segments run in parallel for one (batch, head): enough workgroups
-// to give every CU about two, each segment at least four 64-token steps long.
-// wkv_tune(WKV_TUNE_SEGMENTS) / RWKV_WKV_NSEG override it.
+// How many time segments run in parallel for one (batch, head).  More segments mean
+// more workgroups (B*H*nseg) to spread over the 256 CUs but also one more light pass
+// over the inputs and a longer fold; the estimate below counts CU rounds times steps
+// per segment and prefers fewer segments on ties.  wkv_tune(WKV_TUNE_SEGMENTS) /
+// RWKV_WKV_NSEG override it.
 struct SegPlan { int nseg, sps; };
 inline int &forced_segments() {          // 0 = choose automatically
     static int v = [] { const char *e = getenv("RWKV_WKV_NSEG"); return e ? atoi(e) : 0; }();
@@ -937,8 +939,18 @@ inline int &forced_segments() {          // 0 = choose automatically
 static SegPlan plan_segments(int BH, int Tlen) {
     const int nsb = (Tlen + SB - 1) / SB;
     const int forced = forced_segments();
-    int want = forced > 0 ? forced : (512 + BH - 1) / BH;
-    want = std::max(1, std::min(want, forced > 0 ? nsb : std::max(1, nsb / 4)));
+    int want = 1;
+    if (forced > 0) {
+        want = std::min(forced, nsb);
+    } else {
+        double best = 1e30;
+        for (int cand = 1; cand <= 16 && cand * 4 <= std::max(4, nsb); cand *= 2) {
+            const int sps = (nsb + cand - 1) / cand;
+            const double rounds = (double)((BH * cand + 255) / 256);
+            const double cost = rounds * (sps + 1) * (cand > 1 ? 1.3 : 1.0);
+            if (cost < best * 0.97) { best = cost; want = cand; }
+        }
+    }
     const int sps = (nsb + want - 1) / want;
     return SegPlan{(nsb + sps - 1) / sps, sps};
 }
