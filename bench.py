@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline times")
     ap.add_argument("--rotate", type=int, default=3, help="distinct input sets cycled through")
     ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run three plain 256 MiB device copies first (reference point for the FETCH_SIZE / "
+                         "WRITE_SIZE counters of a profiler run)")
     return ap.parse_args()
 
 
@@ -218,6 +221,17 @@ def cpu_baseline(cfg, heads):
     return out
 
 
+def measured_traffic(cfg, algo, segments, kernel):
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 counter
+    summary of this same workload (profiles/), or None when there is none for it."""
+    path = os.path.join(ROOT, "profiles", f"wkv6_cfg{cfg}_traffic.json")
+    if not os.path.exists(path):
+        return None
+    rec = json.load(open(path))
+    same = rec.get("algo") == algo and rec.get("segments") == (segments or "auto") and rec.get("kernel") == kernel
+    return rec["traffic_bytes_per_launch"] if same else None
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -229,6 +243,12 @@ def main():
     runner = (Runner4 if a.cfg == 2 else Runner56)(a.cfg, a.algo, a.rotate)
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
+    if a.traffic_probe:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     for _ in range(a.warmup):
         runner.step()
     torch.cuda.synchronize()
@@ -251,9 +271,10 @@ def main():
     dom = max(kern, key=lambda k: kern[k]["ms"])
     dom_bytes = runner.bytes_bwd if dom == "backward" else runner.bytes_fwd
     achieved = dom_bytes / (kern[dom]["ms"] * 1e-3) / 1e9
+    kname = f"{dom} (kernel id {kern[dom]['kernel_id']})"
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                "kernel": f"{dom} (kernel id {kern[dom]['kernel_id']})",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(a.cfg, a.algo, a.segments, kname),
+                "kernel": kname,
                 "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_ms": kern[dom]["ms"],
                 "kernels_ms": {k: v["ms"] for k, v in kern.items()},
                 "whole_step_GBs": runner.bytes_step / (ms_step * 1e-3) / 1e9,
