@@ -172,6 +172,8 @@ struct FwdTiles {
     uint16_t vT[SB * LD];    // v                [value][token]
     float dec[4][HEAD];      // e^{b} per block and key
     float rho[SB];           // r . (u o k) per token
+    uint4 amat[4][64];       // the masked intra-block matrix of each block as MFMA A-operand fragments
+                             // (head, remainder), one 16-byte entry per lane; built once, used by all wavefronts
 };
 
 // Forward over one segment (`sps` 64-token steps) of one (batch, head); grid =
@@ -180,8 +182,9 @@ struct FwdTiles {
 //                    summary in `part`;
 //   main pass        (all segments): folds the summaries of the earlier segments
 //                    into s_in to get its own starting state, then produces y.
-// ckpt (optional) receives the state at the start of every 64-token step,
-// [bh][step][key][value] fp32; the last segment writes s_out.
+// ckpt (optional) receives the state at the start of every 64-token step, fp32, in the
+// accumulator layout of this kernel: [bh][step][value/16][key/16][lane][4] with
+// lane = 16*((key%16)/4) + value%16 and the last index = key%4; the last segment writes s_out.
 template <bool PER_TOKEN_W, bool STATE_ONLY>
 __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg, int sps,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
@@ -311,56 +314,72 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
         PT_MARK(1)
         if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
 
-        // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
-        if (!STATE_ONLY && ckpt) {
-            float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD;
+        if (!STATE_ONLY) {
+            if (ckpt) {       // state at the start of this step, 16 bytes per lane and tile
+                float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++)
+                for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+            }
+            // ---------------- wavefront q builds the masked intra-block matrix of block q for everybody:
+            // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n.  Three independent
+            // accumulators (head*head, rem*head, head*rem) shorten the dependency chain.
+            const int row = 16 * wv + n;
+            f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
 #pragma unroll
-                for (int e = 0; e < 4; e++) cp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+            for (int kk = 0; kk < 4; kk += 2) {
+                const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
+                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                a0 = mma2(k0, k1, r0, r1, a0);
+                a1 = mma2(frag(sm.knl, row, ca), frag(sm.knl, row, cb), r0, r1, a1);
+                a2 = mma2(k0, k1, frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), a2);
+            }
+            f4 at = a0 + (a1 + a2);
+            const float rho_t = sm.rho[16 * wv + n];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int s_ = 4 * g + e;
+                at[e] = s_ < n ? at[e] : (s_ == n ? rho_t : 0.f);
+            }
+            uint32_t h0, l0, h1, l1;                        // A[t = n][s = 4g..4g+3] as head + remainder
+            split2(at[0], at[1], h0, l0);
+            split2(at[2], at[3], h1, l1);
+            sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
+            __syncthreads();
         }
+
+        // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
+        const bool full = (sb + 1) * SB <= Tlen;
+        bf16 *ystep = y + base + (size_t)(sb * SB) * C;
+        const unsigned ylane = (unsigned)(4 * g) * C + 16 * wv + n;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             if (sb * SB + 16 * q >= Tlen) break;
             const int row = 16 * q + n;
             const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
             if (!STATE_ONLY) {
-                // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n.  Three
-                // independent accumulators (head*head, rem*head, head*rem) shorten the chain.
-                f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
                 // inter-block part of y: rh S, with S as head + remainder
-                f4 y0 = a0, y1 = a0, y2 = a0;
+                f4 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0;
 #pragma unroll
                 for (int kk = 0; kk < 4; kk += 2) {
                     const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                    const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
                     const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                    const s4 r0l = frag(sm.rhl, row, ca), r1l = frag(sm.rhl, row, cb);
-                    a0 = mma2(k0, k1, r0, r1, a0);
-                    a1 = mma2(frag(sm.knl, row, ca), frag(sm.knl, row, cb), r0, r1, a1);
-                    a2 = mma2(k0, k1, r0l, r1l, a2);
                     s4 s0h, s0l, s1h, s1l;
                     split4(S[kk], s0h, s0l);
                     split4(S[kk + 1], s1h, s1l);
                     y0 = mma2(r0, r1, s0h, s1h, y0);
                     y1 = mma2(r0, r1, s0l, s1l, y1);
-                    y2 = mma2(r0l, r1l, s0h, s1h, y2);
+                    y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
                 }
-                f4 at = a0 + (a1 + a2);
-                const float rho_t = sm.rho[16 * q + n];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int s = 4 * g + e;
-                    at[e] = s < n ? at[e] : (s == n ? rho_t : 0.f);
-                }
-                s4 a_hi, a_lo;                                  // A[t = n][s = 4g..4g+3]
-                split4(at, a_hi, a_lo);
+                const uint4 am = sm.amat[q][lane];
                 f4 yt = y0 + (y1 + y2);
-                yt = mma2(a_hi, a_lo, v_op, v_op, yt);
+                yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
+                if (y) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int t = sb * SB + 16 * q + 4 * g + e;
-                    if (y && t < Tlen) y[base + (size_t)t * C + 16 * wv + n] = bf16{bf16_bits(yt[e])};
+                    for (int e = 0; e < 4; e++) {
+                        const unsigned o = ylane + (unsigned)(16 * q + e) * C;
+                        if (full || sb * SB + 16 * q + 4 * g + e < Tlen) ystep[o] = bf16{bf16_bits(yt[e])};
+                    }
                 }
             }
 #pragma unroll
@@ -591,13 +610,13 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
         if (key_side) {
             // ---------------- rebuild the state at the start of each block: ST[kk][e] = S[key own][value 16kk+4g+e]
             f4 ST[4];
-            {
-                const float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD + own * HEAD;
+            {   // checkpoint in the forward kernel's accumulator layout: element [key][value] sits at
+                // tile (value/16, key/16), lane 16*((key%16)/4) + value%16, component key%4
+                const float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
 #pragma unroll
-                for (int kk = 0; kk < 4; kk++) {
-                    const float4 x = *reinterpret_cast<const float4 *>(cp + 16 * kk + 4 * g);
-                    ST[kk][0] = x.x; ST[kk][1] = x.y; ST[kk][2] = x.z; ST[kk][3] = x.w;
-                }
+                for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) ST[kk][e] = cp[kk * 1024 + e * 4];
             }
             f4 Q1[4];                        // gy S^T per block, taken while S passes by: Q1[q][e] at [token 4g+e][key own]
 #pragma unroll

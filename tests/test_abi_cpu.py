@@ -59,7 +59,7 @@ def test_argument_checks_return_before_any_launch(L):
     need = L.wkv6_backward_workspace(1, 8, 64, 1, 1, 0)
     assert need > 0
     args = [one] * 14
-    assert L.wkv6_backward(null, 1, 8, 64, 1, 1, 0, 0, *args, one, need - 1) == -5
+    assert L.wkv6_backward(null, 1, 8, 64, 1, 1, 1, 0, *args, one, need - 1) == -5   # flags = WKV_FLOOR_DECAY
     assert L.wkv4_forward(null, 0, 8, 64, 0, one, one, one, one, null, one, null, null) == -1
     assert L.wkv4_backward(null, 1, 8, 64, 0, *([one] * 13), one, 0) == -5
     assert L.wkv_cumsum_decay(null, 1, 100, 64, 16, 1, one, null, null, null, null, null) == -1
