@@ -41,7 +41,7 @@ namespace chunked {
 #ifdef WKV_PHASE_TIMING
 #define PT_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}; long long pt_last_ = clock64();
 #define PT_MARK(i) { const long long now_ = clock64(); pt_[i] += now_ - pt_last_; pt_last_ = now_; }
-#define PT_PRINT(name) if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) printf("%s[%d]: stage %lld sync %lld compute %lld sync %lld other %lld aux %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5]);
+#define PT_PRINT(name) if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) printf("%s[%d]: p0 %lld p1 %lld p2 %lld p3 %lld p4 %lld p5 %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5]);
 #else
 #define PT_DECL
 #define PT_MARK(i)
@@ -163,30 +163,34 @@ constexpr int PART = HEAD * HEAD + HEAD;
 
 // ------------------------------------------------------------------- forward --
 struct FwdTiles {
-    uint16_t rh[SB * LD];    // r e^{excl}       [token][key]   bf16 head of the value
-    uint16_t rhl[SB * LD];   //                                 bf16 remainder
-    uint16_t kn[SB * LD];    // k e^{-incl}      [token][key]
-    uint16_t knl[SB * LD];
-    uint16_t khT[SB * LD];   // k e^{b-incl}     [key][token]
-    uint16_t khTl[SB * LD];
+    // the summary pass uses (and allocates) only the part up to `rh`
+    uint16_t khT[SB * LD];   // k e^{b-incl}     [key][token]   bf16 head of the value
+    uint16_t khTl[SB * LD];  //                                 bf16 remainder
     uint16_t vT[SB * LD];    // v                [value][token]
     float dec[4][HEAD];      // e^{b} per block and key
+    uint16_t rh[SB * LD];    // r e^{excl}       [token][key]
+    uint16_t rhl[SB * LD];
+    uint16_t kn[SB * LD];    // k e^{-incl}      [token][key]
+    uint16_t knl[SB * LD];
     float rho[SB];           // r . (u o k) per token
     uint4 amat[4][64];       // the masked intra-block matrix of each block as MFMA A-operand fragments
                              // (head, remainder), one 16-byte entry per lane; built once, used by all wavefronts
 };
+constexpr size_t FWD_PASS_LDS = offsetof(FwdTiles, rh);
 
 // Forward over one segment (`sps` 64-token steps) of one (batch, head); grid =
 // B*H*nseg, 4 wavefronts; wavefront w owns value columns 16w..16w+15 of the state.
-//   STATE_ONLY pass  (segments 0..nseg-2): from a zero state, leaves the segment's
-//                    summary in `part`;
-//   main pass        (all segments): folds the summaries of the earlier segments
-//                    into s_in to get its own starting state, then produces y.
-// ckpt (optional) receives the state at the start of every 64-token step, fp32, in the
+//   STATE_ONLY pass  (segments 0..nseg-2, each cut into `m` pieces of `pps` steps so
+//                    that the pass itself fills the GPU): from a zero state, leaves the
+//                    piece's summary in `part`; fold_forward then turns the summaries
+//                    into the state at the start of every segment;
+//   main pass        (all segments): starts from that state (segment 0: from s_in)
+//                    and produces y.
+// ckpt (optional) receives the state at the start of every 64-token step and, in one more slot, the final state, fp32, in the
 // accumulator layout of this kernel: [bh][step][value/16][key/16][lane][4] with
 // lane = 16*((key%16)/4) + value%16 and the last index = key%4; the last segment writes s_out.
 template <bool PER_TOKEN_W, bool STATE_ONLY>
-__global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg, int sps,
+__global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
         bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, float *__restrict__ part,
@@ -194,12 +198,14 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     FwdTiles &sm = *reinterpret_cast<FwdTiles *>(smem_raw);
-    const int nsegk = STATE_ONLY ? nseg - 1 : nseg;
-    const int bh = blockIdx.x / nsegk, seg = blockIdx.x % nsegk, b = bh / H, h = bh % H;
+    const int units = STATE_ONLY ? (nseg - 1) * m : nseg;       // workgroups per (batch, head)
+    const int bh = blockIdx.x / units, unit = blockIdx.x % units, b = bh / H, h = bh % H;
+    const int seg = STATE_ONLY ? unit / m : unit;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
+    const int sb0 = STATE_ONLY ? seg * sps + (unit % m) * pps : seg * sps;
+    const int sb1 = min(min(nsb, (seg + 1) * sps), STATE_ONLY ? sb0 + pps : nsb);
 
     // state tiles: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]
     f4 S[4], Dacc[4];
@@ -208,22 +214,12 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
         S[kk] = f4{0.f, 0.f, 0.f, 0.f};
         Dacc[kk] = f4{1.f, 1.f, 1.f, 1.f};
     }
-    if (!STATE_ONLY) {
-        const float *sp = s_in + (size_t)bh * HEAD * HEAD;
+    if (!STATE_ONLY) {       // segment 0 starts from s_in, a later one from what fold_forward left
+        const float *sp = seg == 0 ? s_in + (size_t)bh * HEAD * HEAD : part + ((size_t)bh * nseg * m + seg * m - 1) * PART;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
             for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
-        for (int gg = 0; gg < seg; gg++) {           // effect of the earlier segments, in order
-            const float *pp = part + ((size_t)bh * nseg + gg) * PART;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int row = 16 * kk + 4 * g + e;
-                    S[kk][e] = fmaf(pp[HEAD * HEAD + row], S[kk][e], pp[row * HEAD + 16 * wv + n]);
-                }
-        }
     }
     // staging role: block wv of the step, tokens 8*half..8*half+7 of it, channels c0, c0+1
     const int half = lane >> 5, c0 = 2 * (lane & 31);
@@ -316,7 +312,7 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
 
         if (!STATE_ONLY) {
             if (ckpt) {       // state at the start of this step, 16 bytes per lane and tile
-                float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
+                float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + sb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
 #pragma unroll
                 for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
             }
@@ -397,7 +393,7 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
     }
     PT_PRINT(STATE_ONLY ? "fwd-state" : "fwd")
     if (STATE_ONLY) {
-        float *pp = part + ((size_t)bh * nseg + seg) * PART;
+        float *pp = part + ((size_t)bh * nseg * m + unit) * PART;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
@@ -406,12 +402,268 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
                 pp[row * HEAD + 16 * wv + n] = S[kk][e];
                 if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
             }
-    } else if (s_out && seg == nseg - 1) {
-        float *op = s_out + (size_t)bh * HEAD * HEAD;
+    } else if (seg == nseg - 1) {
+        if (ckpt) {       // the final state takes the slot after the last step
+            float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + nsb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+        }
+        if (s_out) {
+            float *op = s_out + (size_t)bh * HEAD * HEAD;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) op[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+        }
+    }
+}
+
+// ------------------------------------------------------- forward, 16 wavefronts --
+// The main forward pass with the work of a 64-token step spread over 16 wavefronts:
+// wavefront (q, wv) produces y for block q (16 tokens), value columns 16wv..16wv+15.
+// Every wavefront holds the state at the step's start and advances its own copy
+// over the q blocks before its own (a few MFMAs per block, far cheaper than the
+// block's own work); the wavefronts of the last block advance once more and hand the
+// state at the step's end to the others through LDS.  Four wavefronts per SIMD keep
+// the vector ALU busy where one wavefront alone cannot issue fast enough.
+//
+// Staging: lane = (token of a block, four channels), a block's running log decay is
+// a prefix sum over the 16 lanes of a DPP row.  Every tile is [token][channel]; the
+// operands that the MFMAs want with the tokens along the contraction (k e^{b-incl}, v)
+// come out of the transposing LDS read of gfx950.
+constexpr int NT_F16 = 1024;
+constexpr int LDT = 80;       // row length of the tiles read through the transposing load: four rows of
+                              // eight dwords each must fall into distinct bank groups (40 dwords = 8 mod 32)
+
+struct Fwd16Tiles {
+    uint16_t rh[SB * LD];     // r e^{excl}       [token][key]  bf16 head / remainder
+    uint16_t rhl[SB * LD];
+    uint16_t kn[SB * LD];     // k e^{-incl}      [token][key]
+    uint16_t knl[SB * LD];
+    uint16_t kh[SB * LDT];    // k e^{b-incl}     [token][key]   (read transposed)
+    uint16_t khl[SB * LDT];
+    uint16_t v[SB * LDT];     // v                [token][value] (read transposed)
+    float dec[4][HEAD];       // e^{b} per block and key
+    float rho[4][SB];         // r . (u o k) per token: partial sums over 16 channels each
+    uint4 amat[4][64];        // masked intra-block matrix of each block as A-operand fragments (head, remainder)
+    float4 hand[4][4][64];    // state at the end of the step, accumulator layout [wv][kk][lane]
+};
+
+__device__ __forceinline__ float row_prefix_sum(float x) {      // inclusive, over the 16 lanes of a DPP row
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));
+    return x;
+}
+// Transposing 8-byte LDS read: with every lane (g, a) of a 16-lane group pointing at
+// tile[row0 + 4g + a/4][col0 + 4(a%4) ..+3], lane (g, n) receives tile[row0 + 4g + i][col0 + n], i = 0..3:
+// an MFMA operand fragment with the rows along the contraction.  `off` = the lane's share of the address.
+__device__ __forceinline__ int tr_lane_offset(int lane, int ld) {
+    const int a = lane & 15, g = lane >> 4;
+    return (4 * g + (a >> 2)) * ld + 4 * (a & 3);
+}
+__device__ __forceinline__ s4 frag_tr(const uint16_t *tile, int off) {
+    typedef s4 __attribute__((address_space(3))) lds_s4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)(tile + off));
+}
+
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int nseg, int sps, int m,
+        const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
+        const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
+        bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, const float *__restrict__ part,
+        int floor_decay)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Fwd16Tiles &sm = *reinterpret_cast<Fwd16Tiles *>(smem_raw);
+    const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
+    const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const int q = w16 >> 2, wv = w16 & 3;
+    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    const int nsb = (Tlen + SB - 1) / SB;
+    const int sb0 = seg * sps, sb1 = min(nsb, (seg + 1) * sps);
+
+    // state at the start of the step: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]
+    f4 S[4];
+    {
+        const float *sp = seg == 0 ? s_in + (size_t)bh * HEAD * HEAD : part + ((size_t)bh * nseg * m + seg * m - 1) * PART;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) op[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+            for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
+    }
+    // staging role: token n of block q, channels c4..c4+3
+    const int c4 = 16 * wv + 4 * g, tok = 16 * q + n;
+    const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
+    float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!PER_TOKEN_W) {
+        const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+        l_const = make_float4(log_decay(w4.x, floor_decay), log_decay(w4.y, floor_decay), log_decay(w4.z, floor_decay),
+                              log_decay(w4.w, floor_decay));
+    }
+    uint2 pr, pk, pv;
+    float4 pw;
+    auto fetch = [&](int sb) {
+        const int t = sb * SB + tok;
+        if (t < Tlen) {
+            const size_t o = base + (size_t)t * C + c4;
+            pr = *reinterpret_cast<const uint2 *>(r + o);
+            pk = *reinterpret_cast<const uint2 *>(k + o);
+            pv = *reinterpret_cast<const uint2 *>(v + o);
+            pw = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+        } else {
+            pr = pk = pv = make_uint2(0u, 0u);
+            pw = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    const int tro = tr_lane_offset(lane, LDT);
+
+    fetch(sb0);
+    PT_DECL
+    for (int sb = sb0; sb < sb1; sb++) {
+        PT_MARK(5)
+        // ---------------- prepare the scaled operands of this lane's token
+        {
+            float l[4] = {pw.x, pw.y, pw.z, pw.w}, inc[4], tot[4];
+            const float rf[4] = {bf_lo(pr.x), bf_hi(pr.x), bf_lo(pr.y), bf_hi(pr.y)};
+            const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
+            const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
+            float rhv[4], knv[4], khv[4], p = 0.f;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                if (PER_TOKEN_W) l[c] = log_decay(l[c], floor_decay);
+                inc[c] = row_prefix_sum(l[c]);
+                tot[c] = __shfl(inc[c], lane | 15);
+                rhv[c] = rf[c] * __expf(inc[c] - l[c]);
+                khv[c] = kf[c] * __expf(tot[c] - inc[c]);
+                knv[c] = n == 15 ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
+                p = fmaf(rf[c] * uf[c], kf[c], p);
+            }
+            uint32_t h0, l0, h1, l1;
+            const int o = tok * LD + c4, ot = tok * LDT + c4;
+            split2(rhv[0], rhv[1], h0, l0); split2(rhv[2], rhv[3], h1, l1);
+            *reinterpret_cast<uint2 *>(&sm.rh[o]) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(&sm.rhl[o]) = make_uint2(l0, l1);
+            split2(knv[0], knv[1], h0, l0); split2(knv[2], knv[3], h1, l1);
+            *reinterpret_cast<uint2 *>(&sm.kn[o]) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(&sm.knl[o]) = make_uint2(l0, l1);
+            split2(khv[0], khv[1], h0, l0); split2(khv[2], khv[3], h1, l1);
+            *reinterpret_cast<uint2 *>(&sm.kh[ot]) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(&sm.khl[ot]) = make_uint2(l0, l1);
+            *reinterpret_cast<uint2 *>(&sm.v[ot]) = pv;
+            if (n == 15) *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+            p += __shfl_xor(p, 16);
+            p += __shfl_xor(p, 32);
+            if (g == 0) sm.rho[wv][tok] = p;
+        }
+        PT_MARK(0)
+        __syncthreads();
+        PT_MARK(1)
+        if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
+
+        if (ckpt && q == 0) {       // state at the start of this step, 16 bytes per lane and tile
+            float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + sb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+        }
+        // one block of the state recurrence: S <- e^{b} o S + (k e^{b-incl})^T v
+        auto advance = [&](int blk) {
+            const s4 v_op = frag_tr(sm.v, tro + (16 * blk) * LDT + 16 * wv);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][16 * kk + 4 * g]);
+                S[kk][0] *= d4.x; S[kk][1] *= d4.y; S[kk][2] *= d4.z; S[kk][3] *= d4.w;
+                S[kk] = mma2(frag_tr(sm.kh, tro + (16 * blk) * LDT + 16 * kk), frag_tr(sm.khl, tro + (16 * blk) * LDT + 16 * kk),
+                             v_op, v_op, S[kk]);
+            }
+        };
+        if (q == wv) {
+            // ---------------- builds the masked intra-block matrix of block q for the wavefronts (q, *):
+            // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n
+            const int row = 16 * q + n;
+            f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
+                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                a0 = mma2(k0, k1, r0, r1, a0);
+                a1 = mma2(frag(sm.knl, row, ca), frag(sm.knl, row, cb), r0, r1, a1);
+                a2 = mma2(k0, k1, frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), a2);
+            }
+            f4 at = a0 + (a1 + a2);
+            const float rho_t = (sm.rho[0][row] + sm.rho[1][row]) + (sm.rho[2][row] + sm.rho[3][row]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int s_ = 4 * g + e;
+                at[e] = s_ < n ? at[e] : (s_ == n ? rho_t : 0.f);
+            }
+            uint32_t h0, l0, h1, l1;                        // A[t = n][s = 4g..4g+3] as head + remainder
+            split2(at[0], at[1], h0, l0);
+            split2(at[2], at[3], h1, l1);
+            sm.amat[q][lane] = make_uint4(h0, h1, l0, l1);
+        }
+        // the state at the start of block q (wave-uniform trip count)
+        for (int blk = 0; blk < q; blk++) advance(blk);
+        PT_MARK(2)
+        __syncthreads();
+        PT_MARK(3)
+
+        // ---------------- y of block q, value columns 16wv..16wv+15
+        if (y && sb * SB + 16 * q < Tlen) {
+            const int row = 16 * q + n;
+            f4 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                s4 s0h, s0l, s1h, s1l;
+                split4(S[kk], s0h, s0l);
+                split4(S[kk + 1], s1h, s1l);
+                y0 = mma2(r0, r1, s0h, s1h, y0);
+                y1 = mma2(r0, r1, s0l, s1l, y1);
+                y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
+            }
+            const uint4 am = sm.amat[q][lane];
+            const s4 v_op = frag_tr(sm.v, tro + (16 * q) * LDT + 16 * wv);
+            f4 yt = y0 + (y1 + y2);
+            yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
+            bf16 *yp = y + base + (size_t)(sb * SB + 16 * q + 4 * g) * C + 16 * wv + n;
+            const int left = Tlen - (sb * SB + 16 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (e < left) yp[(size_t)e * C] = bf16{bf16_bits(yt[e])};
+        }
+        if (q == 3) {         // on to the end of the step, for everybody
+            advance(3);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) sm.hand[wv][kk][lane] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+        }
+        PT_MARK(4)
+        __syncthreads();
+        if (q != 3) {
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const float4 x = sm.hand[wv][kk][lane];
+                S[kk] = f4{x.x, x.y, x.z, x.w};
+            }
+        }
+    }
+    PT_PRINT("fwd16")
+    if (seg == nseg - 1 && q == 3) {
+        if (ckpt) {       // the final state takes the slot after the last step
+            float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + nsb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+        }
+        if (s_out) {
+            float *op = s_out + (size_t)bh * HEAD * HEAD;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) op[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+        }
     }
 }
 
@@ -458,7 +710,7 @@ struct BwdTiles {
 };
 
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nseg, int sps,
+__global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
         const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
@@ -481,7 +733,9 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
     // value side: G[kk][e] = G[key 16kk+4g+e][value own]
     f4 G[4];
     {
-        const float *gp = gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr;
+        // the last segment starts from gs_out, an earlier one from what fold_backward left
+        const float *gp = seg == nseg - 1 ? (gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr)
+                                          : gpart + ((size_t)bh * nseg * m + (seg + 1) * m) * PART;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
 #pragma unroll
@@ -489,18 +743,6 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
                 const int x = 16 * kk + 4 * g + e;
                 G[kk][e] = gp ? (key_side ? gp[own * HEAD + x] : gp[x * HEAD + own]) : 0.f;
             }
-        for (int gg = nseg - 1; gg > seg; gg--) {      // effect of the later segments, last first
-            const float *pp = gpart + ((size_t)bh * nseg + gg) * PART;
-            const float d_own = pp[HEAD * HEAD + own];
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int x = 16 * kk + 4 * g + e;
-                    G[kk][e] = key_side ? fmaf(d_own, G[kk][e], pp[own * HEAD + x])
-                                        : fmaf(pp[HEAD * HEAD + x], G[kk][e], pp[x * HEAD + own]);
-                }
-        }
     }
     float A_run = 0.f, gu_acc = 0.f, gw_acc = 0.f;
 
@@ -612,7 +854,7 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
             f4 ST[4];
             {   // checkpoint in the forward kernel's accumulator layout: element [key][value] sits at
                 // tile (value/16, key/16), lane 16*((key%16)/4) + value%16, component key%4
-                const float *cp = ckpt + ((size_t)bh * nsb + sb) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
+                const float *cp = ckpt + ((size_t)bh * (nsb + 1) + sb) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
 #pragma unroll
                 for (int kk = 0; kk < 4; kk++)
 #pragma unroll
@@ -832,11 +1074,12 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
     }
 }
 
-// State-gradient summary of one segment (segments 1..nseg-1) for the backward
-// split: from a zero gradient, walks the segment's tokens last to first with
+// State-gradient summary of one piece (`pps` steps) of the segments 1..nseg-1 for the
+// backward split: from a zero gradient, walks the piece's tokens last to first with
 //   G <- e^{b} o G + (r e^{excl})^T gy      per 16-token block
-// and leaves  delta = G, decay = product of e^{b}  in gpart.  One wavefront per
-// 16 value columns, as the forward's state.
+// and leaves  delta = G, decay = product of e^{b}  in gpart; fold_backward turns the
+// summaries into the gradient at the end of every segment.  One wavefront per 16 value
+// columns, as the forward's state.
 struct GPassTiles {
     uint16_t rhT[SB * LD];   // r e^{excl}   [key][token]  head / remainder
     uint16_t rhTl[SB * LD];
@@ -845,16 +1088,17 @@ struct GPassTiles {
 };
 
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, int nseg, int sps,
+__global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
         const bf16 *__restrict__ r, const float *__restrict__ wraw, const bf16 *__restrict__ gy,
         float *__restrict__ gpart, int floor_decay)
 {
     __shared__ __align__(16) GPassTiles sm;
-    const int bh = blockIdx.x / (nseg - 1), seg = 1 + blockIdx.x % (nseg - 1), b = bh / H, h = bh % H;
+    const int units = (nseg - 1) * m;
+    const int bh = blockIdx.x / units, piece = m + blockIdx.x % units, seg = piece / m, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
+    const int sb0 = seg * sps + (piece % m) * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
     const int half = lane >> 5, c0 = 2 * (lane & 31);
     float2 l_const = make_float2(0.f, 0.f);
     if (!PER_TOKEN_W) {
@@ -929,7 +1173,7 @@ __global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, in
         }
         __syncthreads();
     }
-    float *pp = gpart + ((size_t)bh * nseg + seg) * PART;
+    float *pp = gpart + ((size_t)bh * nseg * m + piece) * PART;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
 #pragma unroll
@@ -940,9 +1184,496 @@ __global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, in
         }
 }
 
+// ------------------------------------------------------ backward, 16 wavefronts --
+// The same mathematics as `backward`, with the work of a 64-token step spread over 16
+// wavefronts (four per SIMD) so that no single wavefront's instruction stream is the
+// critical path.  A step runs in three phases separated by workgroup barriers:
+//
+//   prepare   all wavefronts: lane = (token of a block, four channels), every tile is
+//             [token][channel]; fragments with the tokens along the contraction come
+//             from the transposing LDS read.
+//   chains    wavefronts  0-3  walk the state forward from the step's checkpoint and
+//                              leave  Q1 = gy S^T  of each block in LDS;
+//             wavefronts  4-7  walk the state gradient backward (value-major copy) and
+//                              leave  Q4 = v G^T;
+//             wavefronts  8-11 walk the key-major copy and keep  kh G  in registers;
+//             wavefronts 12-15 build, per block, the masked matrices P, P^T and A~ once
+//                              for everybody.
+//   blocks    wavefront (q, w): gr, gk and the decay gradient of block q, keys
+//             16w..16w+15; wavefronts 8-11 also finish gv.
+//
+// The running sum of the decay gradient is anchored once per segment (at the segment's
+// end, from the state checkpoint there and the gradient handed in) and carried from
+// step to step in LDS; inside a step every block sums its own tokens and the blocks
+// are joined through LDS.
+struct Bwd16Tiles {
+    uint16_t gy[SB * LD];    // gy              [token][value]
+    uint16_t v[SB * LD];     // v               [token][value]
+    uint16_t rh[SB * LD];    // r e^{excl}      [token][key]   head / remainder
+    uint16_t rhl[SB * LD];
+    uint16_t kn[SB * LD];    // k e^{-incl}     [token][key]
+    uint16_t knl[SB * LD];
+    uint16_t kh[SB * LD];    // k e^{b-incl}    [token][key]
+    uint16_t khl[SB * LD];
+    float incl[SB * HEAD];   // inclusive running log decay inside the block [token][key]
+    float lw[SB * HEAD];     // log w                                         [token][key]
+    float tot[4][HEAD];      // b per block and key
+    float dec[4][HEAD];      // e^{b}
+    float rho[4][SB];        // r . (u o k) per token: partial sums over 16 channels each
+    float q1[SB * HEAD];     // gy S^T          [token][key]
+    float q4[SB * HEAD];     // v G^T           [token][key]
+    uint4 pfr[4][2][64];     // per block: P^T masked to s < t, P masked to t > s, as A-operand fragments (head, remainder)
+    float pdiag[4][16];      // P[t][t]
+    uint4 amat[4][64];       // A~ masked to t >= s (diagonal r.(u o k)), A-operand fragments (head, remainder)
+    float tots[4][HEAD];     // per block and key: sum over the block's tokens of r gr - k gk
+    float arun[HEAD];        // the running sum at the end of the current step
+    float red[2][4][HEAD];   // gu / gw partial sums of the four block groups
+};
+constexpr int NT_B16 = 1024;
+// Re-derives the lane-dependent indices from an opaque copy of the lane id, so that the
+// address arithmetic of a phase stays inside the phase instead of being hoisted out of the
+// step loop into registers that live (and spill) across the whole kernel.
+#define WKV_LOCAL_LANE                                                                                        \
+    int lane_v_ = lane0;                                                                                      \
+    asm volatile("" : "+v"(lane_v_));                                                                         \
+    const int lane = lane_v_, g = lane >> 4, n = lane & 15, own = 16 * wv + n, c4 = 16 * wv + 4 * g,           \
+              tok = 16 * q + n, tro = tr_lane_offset(lane, LD);                                               \
+    (void)tro; (void)c4; (void)tok; (void)own;
+
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int nseg, int sps, int m,
+        const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
+        const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
+        const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
+        bf16 *__restrict__ gr, bf16 *__restrict__ gk, bf16 *__restrict__ gv, float *__restrict__ gw_tok,
+        float *__restrict__ gw_part, float *__restrict__ gu_part, float *__restrict__ gs_in, int floor_decay)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Bwd16Tiles &sm = *reinterpret_cast<Bwd16Tiles *>(smem_raw);
+    const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
+    const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const int role = w16 >> 2, q = role, wv = w16 & 3;      // chain role; block (for preparing and for the block phase); quarter
+    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    const int nsb = (Tlen + SB - 1) / SB;
+    const int sb0 = seg * sps, sb1 = min(nsb, (seg + 1) * sps);
+    const int own = 16 * wv + n;               // key (or, for the key-major gradient, value) channel of this lane
+    const float u_i = u[h * HEAD + own];
+    const float *ck_lane = ckpt + (size_t)bh * (nsb + 1) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
+
+    // One register tile set per wavefront, by role:
+    //   wavefronts 0-3:   the state,   G[kk][e] = S[key own][value 16kk+4g+e]  (reloaded from the checkpoint every step)
+    //   wavefronts 4-7:   its gradient, G[kk][e] = G[key own][value 16kk+4g+e]
+    //   wavefronts 8-11:  its gradient, G[kk][e] = G[key 16kk+4g+e][value own]
+    f4 G[4] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
+    {
+        // the last segment starts from gs_out, an earlier one from what fold_summaries left
+        const float *gp = seg == nseg - 1 ? (gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr)
+                                          : gpart + ((size_t)bh * nseg * m + (seg + 1) * m) * PART;
+        if (gp && (role == 1 || role == 2)) {
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int x = 16 * kk + 4 * g + e;
+                    G[kk][e] = role == 1 ? gp[own * HEAD + x] : gp[x * HEAD + own];
+                }
+        }
+        if (role == 0) {       // anchor of the decay-gradient sum at the segment's end: sum_j G o S
+            float a = 0.f;
+            if (gp) {
+                const float *cp = ck_lane + (size_t)sb1 * HEAD * HEAD;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) a = fmaf(gp[own * HEAD + 16 * kk + 4 * g + e], cp[kk * 1024 + e * 4], a);
+            }
+            a = group_sum4(a);
+            if (g == 0) sm.arun[own] = a;
+        }
+    }
+    float gu_acc = 0.f, gw_acc = 0.f;
+
+    // preparing role: token n of block q, channels c4..c4+3
+    const int c4 = 16 * wv + 4 * g, tok = 16 * q + n;
+    float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!PER_TOKEN_W) {
+        const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+        l_const = make_float4(log_decay(w4.x, floor_decay), log_decay(w4.y, floor_decay), log_decay(w4.z, floor_decay),
+                              log_decay(w4.w, floor_decay));
+    }
+    uint2 pr, pk, pv, pg;
+    float4 pw;
+    auto fetch = [&](int sb, int tok, int c4) {       // (tok, c4 handed in: see WKV_LOCAL_LANE)
+        const int t = sb * SB + tok;
+        if (t < Tlen) {
+            const size_t o = base + (size_t)t * C + c4;
+            pr = *reinterpret_cast<const uint2 *>(r + o);
+            pk = *reinterpret_cast<const uint2 *>(k + o);
+            pv = *reinterpret_cast<const uint2 *>(v + o);
+            pg = *reinterpret_cast<const uint2 *>(gy + o);
+            pw = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+        } else {
+            pr = pk = pv = pg = make_uint2(0u, 0u);
+            pw = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    const int lane0 = lane;
+
+    fetch(sb1 - 1, tok, c4);
+    PT_DECL
+    for (int sb = sb1 - 1; sb >= sb0; sb--) {
+      PT_MARK(5)
+      {
+        WKV_LOCAL_LANE
+        // the step's checkpoint: loads issued now are back when the chains start
+        if (role == 0) {
+            const float *ck_lane = ckpt + (size_t)bh * (nsb + 1) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
+            const float *cp = ck_lane + (size_t)sb * HEAD * HEAD;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) G[kk][e] = cp[kk * 1024 + e * 4];
+        }
+        // ---------------- prepare the operands of this lane's token
+        {
+            float l[4] = {pw.x, pw.y, pw.z, pw.w}, inc[4], tot[4];
+            const float rf[4] = {bf_lo(pr.x), bf_hi(pr.x), bf_lo(pr.y), bf_hi(pr.y)};
+            const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
+            const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
+            const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
+            float rhv[4], knv[4], khv[4], p = 0.f;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                if (PER_TOKEN_W) l[c] = log_decay(l[c], floor_decay);
+                inc[c] = row_prefix_sum(l[c]);
+                tot[c] = __shfl(inc[c], lane | 15);
+                rhv[c] = rf[c] * __expf(inc[c] - l[c]);
+                khv[c] = kf[c] * __expf(tot[c] - inc[c]);
+                knv[c] = n == 15 ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
+                p = fmaf(rf[c] * uf[c], kf[c], p);
+            }
+            uint32_t h0, l0, h1, l1;
+            const int o = tok * LD + c4;
+            *reinterpret_cast<uint2 *>(&sm.gy[o]) = pg;
+            *reinterpret_cast<uint2 *>(&sm.v[o]) = pv;
+            split2(rhv[0], rhv[1], h0, l0); split2(rhv[2], rhv[3], h1, l1);
+            *reinterpret_cast<uint2 *>(&sm.rh[o]) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(&sm.rhl[o]) = make_uint2(l0, l1);
+            split2(knv[0], knv[1], h0, l0); split2(knv[2], knv[3], h1, l1);
+            *reinterpret_cast<uint2 *>(&sm.kn[o]) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(&sm.knl[o]) = make_uint2(l0, l1);
+            split2(khv[0], khv[1], h0, l0); split2(khv[2], khv[3], h1, l1);
+            *reinterpret_cast<uint2 *>(&sm.kh[o]) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(&sm.khl[o]) = make_uint2(l0, l1);
+            *reinterpret_cast<float4 *>(&sm.incl[tok * HEAD + c4]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
+            *reinterpret_cast<float4 *>(&sm.lw[tok * HEAD + c4]) = make_float4(l[0], l[1], l[2], l[3]);
+            if (n == 15) {
+                *reinterpret_cast<float4 *>(&sm.tot[q][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
+                *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+            }
+            p += __shfl_xor(p, 16);
+            p += __shfl_xor(p, 32);
+            if (g == 0) sm.rho[wv][tok] = p;
+        }
+      }
+        PT_MARK(0)
+        __syncthreads();
+        PT_MARK(1)
+
+        f4 KG[4];                    // wavefronts 8-11: kh G per block, KG[q][e] at [token 4g+e][value own]
+      {
+        WKV_LOCAL_LANE
+        if (sb > sb0) fetch(sb - 1, tok, c4);
+        if (role == 0) {
+            // ---------------- state chain, first block to last; Q1[t][key own] = sum_j gy[t][j] S[key own][j]
+#pragma unroll
+            for (int qq = 0; qq < 4; qq++) {
+                f4 qa = {0.f, 0.f, 0.f, 0.f}, qb = qa;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk += 2) {
+                    s4 s0h, s0l, s1h, s1l;
+                    split4(G[kk], s0h, s0l);
+                    split4(G[kk + 1], s1h, s1l);
+                    const s4 y0 = frag(sm.gy, 16 * qq + n, 16 * kk + 4 * g), y1 = frag(sm.gy, 16 * qq + n, 16 * kk + 16 + 4 * g);
+                    qa = mma2(y0, y1, s0h, s1h, qa);
+                    qb = mma2(y0, y1, s0l, s1l, qb);
+                }
+                qa += qb;
+#pragma unroll
+                for (int e = 0; e < 4; e++) sm.q1[(16 * qq + 4 * g + e) * HEAD + own] = qa[e];
+                if (qq < 3) {
+                    const float dq = sm.dec[qq][own];
+                    const s4 khf = frag_tr(sm.kh, tro + (16 * qq) * LD + 16 * wv), khfl = frag_tr(sm.khl, tro + (16 * qq) * LD + 16 * wv);
+#pragma unroll
+                    for (int kk = 0; kk < 4; kk++) {
+                        G[kk] = G[kk] * dq;
+                        const s4 vf_ = frag_tr(sm.v, tro + (16 * qq) * LD + 16 * kk);
+                        G[kk] = mma2(vf_, vf_, khf, khfl, G[kk]);
+                    }
+                }
+            }
+        } else if (role == 1) {
+            // ---------------- state-gradient chain (value-major), last block to first; Q4[s][key own] = sum_j v[s][j] G[key own][j]
+#pragma unroll
+            for (int qq = 3; qq >= 0; qq--) {
+                f4 q4 = {0.f, 0.f, 0.f, 0.f}, q4b = q4;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk += 2) {
+                    s4 g0h, g0l, g1h, g1l;
+                    split4(G[kk], g0h, g0l);
+                    split4(G[kk + 1], g1h, g1l);
+                    const s4 v0 = frag(sm.v, 16 * qq + n, 16 * kk + 4 * g), v1 = frag(sm.v, 16 * qq + n, 16 * kk + 16 + 4 * g);
+                    q4 = mma2(v0, v1, g0h, g1h, q4);
+                    q4b = mma2(v0, v1, g0l, g1l, q4b);
+                }
+                q4 += q4b;
+#pragma unroll
+                for (int e = 0; e < 4; e++) sm.q4[(16 * qq + 4 * g + e) * HEAD + own] = q4[e];
+                const float dq = sm.dec[qq][own];
+                const s4 rhTf = frag_tr(sm.rh, tro + (16 * qq) * LD + 16 * wv), rhTfl = frag_tr(sm.rhl, tro + (16 * qq) * LD + 16 * wv);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {      // G <- e^{b} o G + rh^T gy
+                    G[kk] = G[kk] * dq;
+                    const s4 gT_ = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * kk);
+                    G[kk] = mma2(gT_, gT_, rhTf, rhTfl, G[kk]);
+                }
+            }
+        } else if (role == 2) {
+            // ---------------- state-gradient chain (key-major), last block to first; KG[s][value own] = sum_i kh[s][i] G[i][value own]
+#pragma unroll
+            for (int qq = 3; qq >= 0; qq--) {
+                const int row = 16 * qq + n;
+                f4 g0 = {0.f, 0.f, 0.f, 0.f}, g1 = g0, g2 = g0;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk += 2) {
+                    const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                    s4 g0h, g0l, g1h, g1l;
+                    split4(G[kk], g0h, g0l);
+                    split4(G[kk + 1], g1h, g1l);
+                    const s4 h0 = frag(sm.kh, row, ca), h1 = frag(sm.kh, row, cb);
+                    g0 = mma2(h0, h1, g0h, g1h, g0);
+                    g1 = mma2(h0, h1, g0l, g1l, g1);
+                    g2 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g2);
+                }
+                KG[qq] = g0 + (g1 + g2);
+                const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {      // G <- e^{b} o G + rh^T gy
+                    const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[qq][16 * kk + 4 * g]);
+                    G[kk][0] *= d4.x; G[kk][1] *= d4.y; G[kk][2] *= d4.z; G[kk][3] *= d4.w;
+                    G[kk] = mma2(frag_tr(sm.rh, tro + (16 * qq) * LD + 16 * kk), frag_tr(sm.rhl, tro + (16 * qq) * LD + 16 * kk),
+                                 gyTf, gyTf, G[kk]);
+                }
+                __builtin_amdgcn_sched_barrier(0);      // one block at a time: keeps the register need of the chain bounded
+            }
+        } else {
+            // ---------------- the masked matrices of block wv, once for everybody
+            const int row = 16 * wv + n;
+            s4 gyf[4], vf[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                gyf[kk] = frag(sm.gy, row, 16 * kk + 4 * g);
+                vf[kk] = frag(sm.v, row, 16 * kk + 4 * g);
+            }
+            // pt[e] = P[t = 4g+e][s = n],  ptT[e] = P[t = n][s = 4g+e],  P[t][s] = gy_t . v_s
+            f4 pt = {0.f, 0.f, 0.f, 0.f}, ptT = pt;
+            pt = mma2(gyf[0], gyf[1], vf[0], vf[1], pt);
+            ptT = mma2(vf[0], vf[1], gyf[0], gyf[1], ptT);
+            pt = mma2(gyf[2], gyf[3], vf[2], vf[3], pt);
+            ptT = mma2(vf[2], vf[3], gyf[2], gyf[3], ptT);
+            f4 pm, pTm;
+            {
+                const int e_diag = n & 3;
+                if ((n >> 2) == g) sm.pdiag[wv][n] = e_diag == 0 ? pt[0] : e_diag == 1 ? pt[1] : e_diag == 2 ? pt[2] : pt[3];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int x = 4 * g + e;
+                    pm[e] = x > n ? pt[e] : 0.f;        // later tokens t > s
+                    pTm[e] = x < n ? ptT[e] : 0.f;      // earlier tokens s < t
+                }
+                uint32_t h0, l0, h1, l1;
+                split2(pTm[0], pTm[1], h0, l0); split2(pTm[2], pTm[3], h1, l1);
+                sm.pfr[wv][0][lane] = make_uint4(h0, h1, l0, l1);
+                split2(pm[0], pm[1], h0, l0); split2(pm[2], pm[3], h1, l1);
+                sm.pfr[wv][1][lane] = make_uint4(h0, h1, l0, l1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // A~[t = 4g+e][s = n] = rh_t . kn_s
+            f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
+#pragma unroll
+            for (int kk = 0; kk < 4; kk += 2) {
+                const int ca = 16 * kk + 4 * g, cb = ca + 16;
+                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
+                a0 = mma2(r0, r1, k0, k1, a0);
+                a1 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), k0, k1, a1);
+                a2 = mma2(r0, r1, frag(sm.knl, row, ca), frag(sm.knl, row, cb), a2);
+            }
+            f4 at = a0 + (a1 + a2);
+            const float rho_s = (sm.rho[0][row] + sm.rho[1][row]) + (sm.rho[2][row] + sm.rho[3][row]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int x = 4 * g + e;
+                at[e] = x > n ? at[e] : (x == n ? rho_s : 0.f);
+            }
+            uint32_t h0, l0, h1, l1;
+            split2(at[0], at[1], h0, l0); split2(at[2], at[3], h1, l1);
+            sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
+        }
+      }
+        PT_MARK(2)
+        __syncthreads();
+        PT_MARK(3)
+
+        float Dloc[4], lfac[4];
+      {
+        WKV_LOCAL_LANE
+        if (role == 2) {
+            // ---------------- gv[s][value own] = kh G + sum_{t>=s} A~[t][s] gy[t]
+#pragma unroll
+            for (int qq = 0; qq < 4; qq++) {
+                const uint4 am = sm.amat[qq][lane];
+                const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
+                const f4 gvt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), gyTf, gyTf, KG[qq]);
+                bf16 *gp = gv + base + (size_t)(sb * SB + 16 * qq + 4 * g) * C + own;
+                const int left = Tlen - (sb * SB + 16 * qq + 4 * g);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (e < left) gp[(size_t)e * C] = bf16{bf16_bits(gvt[e])};
+            }
+        }
+        // ---------------- block q, keys 16wv..16wv+15: gr, gk, decay gradient
+        {
+            const uint4 pa = sm.pfr[q][0][lane], pb = sm.pfr[q][1][lane];
+            const s4 pT_h = as_s4(pa.x, pa.y), pT_l = as_s4(pa.z, pa.w), pm_h = as_s4(pb.x, pb.y), pm_l = as_s4(pb.z, pb.w);
+            const s4 khTf = frag_tr(sm.kh, tro + (16 * q) * LD + 16 * wv), khTfl = frag_tr(sm.khl, tro + (16 * q) * LD + 16 * wv);
+            const s4 rhTf = frag_tr(sm.rh, tro + (16 * q) * LD + 16 * wv), rhTfl = frag_tr(sm.rhl, tro + (16 * q) * LD + 16 * wv);
+            f4 q2 = {0.f, 0.f, 0.f, 0.f}, q2b = q2, q3 = q2, q3b = q2;
+            q2 = mma2(pT_h, pT_l, khTf, khTf, q2);      // sum_{s<t} P[t][s] kh_s
+            q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);      // sum_{t>s} P[t][s] rh_t
+            q2b = mma(pT_h, khTfl, q2b);
+            q3b = mma(pm_h, rhTfl, q3b);
+            q2 += q2b; q3 += q3b;
+            const float tot_i = sm.tot[q][own], ent_i = __expf(-tot_i);
+            float c[4], z[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int tk = 16 * q + 4 * g + e;
+                const int t = sb * SB + tk;
+                const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
+                const float E1 = __expf(exc), E2 = __expf(tot_i - inc);
+                const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
+                // r, k back from their scaled head + remainder (16 mantissa bits)
+                const float rr = (bf2f(sm.rh[tk * LD + own]) + bf2f(sm.rhl[tk * LD + own])) * __expf(-exc);
+                const float kr = (bf2f(sm.kh[tk * LD + own]) + bf2f(sm.khl[tk * LD + own])) * __expf(inc - tot_i);
+                const float grv = E1 * (q1 + ent_i * q2[e]) + u_i * kr * pd;
+                const float gkn = E2 * (ent_i * q3[e] + q4);
+                const float gkv = gkn + u_i * rr * pd;
+                c[e] = rr * grv - kr * gkv;
+                z[e] = kr * gkn;
+                lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
+                gu_acc = fmaf(rr * kr, pd, gu_acc);
+                if (t < Tlen) {
+                    const size_t o = base + (size_t)t * C;
+                    gr[o + own] = bf16{bf16_bits(grv)};
+                    gk[o + own] = bf16{bf16_bits(gkv)};
+                }
+            }
+            // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over the block's later tokens of c
+            const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
+            const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
+            const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
+            const float all = group_sum4(mine);
+            Dloc[0] = later + suf0 - z[0];
+            Dloc[1] = later + suf1 - z[1];
+            Dloc[2] = later + suf2 - z[2];
+            Dloc[3] = later - z[3];
+            if (g == 0) sm.tots[q][own] = all;
+        }
+      }
+        PT_MARK(4)
+        __syncthreads();
+        {
+            WKV_LOCAL_LANE
+            float A_end = sm.arun[own];          // at the end of block q: the step's end plus the later blocks
+#pragma unroll
+            for (int qq = 3; qq >= 1; qq--) A_end += qq > q ? sm.tots[qq][own] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int t = sb * SB + 16 * q + 4 * g + e;
+                const float Dt = A_end + Dloc[e];
+                if (PER_TOKEN_W) {
+                    if (t < Tlen) gw_tok[base + (size_t)t * C + own] = Dt * lfac[e];
+                } else {
+                    gw_acc += (t < Tlen) ? Dt : 0.f;
+                }
+            }
+        }
+        __syncthreads();
+        if (role == 0 && g == 0) sm.arun[own] += (sm.tots[0][own] + sm.tots[1][own]) + (sm.tots[2][own] + sm.tots[3][own]);
+    }
+
+    PT_PRINT("bwd16")
+    if (role == 1 && gs_in && seg == 0) {
+        float *gp = gs_in + (size_t)bh * HEAD * HEAD + own * HEAD;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+            *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(G[kk][0], G[kk][1], G[kk][2], G[kk][3]);
+    }
+    gu_acc = group_sum4(gu_acc);
+    gw_acc = group_sum4(gw_acc);
+    if (g == 0) {
+        sm.red[0][q][own] = gu_acc;
+        sm.red[1][q][own] = gw_acc;
+    }
+    __syncthreads();
+    if (q == 0 && g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
+        const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
+        gu_part[po] = (sm.red[0][0][own] + sm.red[0][1][own]) + (sm.red[0][2][own] + sm.red[0][3][own]);
+        if (!PER_TOKEN_W) {
+            bool fl;
+            const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
+            gw_part[po] = fl ? 0.f : ((sm.red[1][0][own] + sm.red[1][1][own]) + (sm.red[1][2][own] + sm.red[1][3][own])) * l;
+        }
+    }
+}
+
+// Chains the piece summaries (S_out = decay o S_in + delta, one decay per key) of one
+// (batch, head) in order, one lane per state element.  `first`..`last` are the pieces
+// the pass produced; going up (forward, step = +1) it starts from `start` and leaves
+// the state at the start of segment s in the slot of piece s*m - 1; going down
+// (backward, step = -1) it leaves the gradient at the end of segment s in the slot of
+// piece (s+1)*m.  In place: a slot is overwritten by the lane that has just read it.
+__global__ __launch_bounds__(256) void fold_summaries(int first, int last, int step, int m, int stride,
+        const float *__restrict__ start, float *__restrict__ part)
+{
+    const int bh = blockIdx.x / (HEAD * HEAD / 256), el = (blockIdx.x % (HEAD * HEAD / 256)) * 256 + threadIdx.x;
+    const int key = el / HEAD;
+    float *pp = part + (size_t)bh * stride * PART;
+    float S = start ? start[(size_t)bh * HEAD * HEAD + el] : 0.f;
+    const int count = (last - first) * step + 1;
+    for (int i0 = 0; i0 < count; i0 += 4) {        // four loads in flight per lane
+        float dl[4], dd[4];
+#pragma unroll
+        for (int x = 0; x < 4; x++)
+            if (i0 + x < count) {
+                const float *q = pp + (size_t)(first + (i0 + x) * step) * PART;
+                dl[x] = q[el];
+                dd[x] = q[HEAD * HEAD + key];
+            }
+#pragma unroll
+        for (int x = 0; x < 4; x++)
+            if (i0 + x < count) {
+                const int piece = first + (i0 + x) * step;
+                S = fmaf(dd[x], S, dl[x]);
+                if (step > 0 ? (piece + 1) % m == 0 : piece % m == 0) pp[(size_t)piece * PART + el] = S;
+            }
+    }
+}
+
 // ------------------------------------------------------------------ launchers --
 size_t checkpoint_bytes(int B, int Tlen, int H) {
-    return (size_t)B * H * ((Tlen + SB - 1) / SB) * HEAD * HEAD * sizeof(float);
+    return (size_t)B * H * ((Tlen + SB - 1) / SB + 1) * HEAD * HEAD * sizeof(float);     // one slot per step + the final state
 }
 
 // How many time segments run in parallel for one (batch, head).  More segments mean
@@ -950,9 +1681,14 @@ size_t checkpoint_bytes(int B, int Tlen, int H) {
 // over the inputs and a longer fold; the estimate below counts CU rounds times steps
 // per segment and prefers fewer segments on ties.  wkv_tune(WKV_TUNE_SEGMENTS) /
 // RWKV_WKV_NSEG override it.
-struct SegPlan { int nseg, sps; };
+constexpr int MAX_SEG = 64;
+struct SegPlan { int nseg, sps, m, pps; };     // segments, steps per segment, pieces per segment, steps per piece
 inline int &forced_segments() {          // 0 = choose automatically
     static int v = [] { const char *e = getenv("RWKV_WKV_NSEG"); return e ? atoi(e) : 0; }();
+    return v;
+}
+inline int &forced_piece_steps() {       // 0 = choose automatically
+    static int v = [] { const char *e = getenv("RWKV_WKV_PPS"); return e ? atoi(e) : 0; }();
     return v;
 }
 static SegPlan plan_segments(int BH, int Tlen) {
@@ -971,9 +1707,18 @@ static SegPlan plan_segments(int BH, int Tlen) {
         }
     }
     const int sps = (nsb + want - 1) / want;
-    return SegPlan{(nsb + sps - 1) / sps, sps};
+    const int nseg = (nsb + sps - 1) / sps;
+    // the summary pass: cut each segment into pieces until the pass has two workgroups per CU
+    // (every piece costs one 16 KB summary, so no finer than needed and never below 2 steps)
+    int pps = sps;
+    if (nseg == 1) return SegPlan{1, sps, 1, sps};
+    if (forced_piece_steps() > 0) pps = std::min(sps, forced_piece_steps());
+    else
+        while (pps >= 4 && (long)BH * (nseg - 1) * ((sps + pps - 1) / pps) < 512) pps = (pps + 1) / 2;
+    int m = (sps + pps - 1) / pps;
+    if (nseg * m > MAX_SEG) { m = std::max(1, MAX_SEG / nseg); pps = (sps + m - 1) / m; m = (sps + pps - 1) / pps; }
+    return SegPlan{nseg, sps, m, pps};
 }
-constexpr int MAX_SEG = 64;
 static size_t part_bytes(int B, int H) { return (size_t)B * H * MAX_SEG * PART * sizeof(float); }
 
 // workspace of a forward call: checkpoints | forward segment summaries
@@ -994,37 +1739,40 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
                           void *workspace, bool keep_ckpt, int floor_decay) {
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = allow_lds(forward<true, false>, sizeof(FwdTiles));
-        if (e == hipSuccess) e = allow_lds(forward<false, false>, sizeof(FwdTiles));
-        if (e == hipSuccess) e = allow_lds(forward<true, true>, sizeof(FwdTiles));
-        if (e == hipSuccess) e = allow_lds(forward<false, true>, sizeof(FwdTiles));
+        hipError_t e = allow_lds(forward16<true>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow_lds(forward16<false>, sizeof(Fwd16Tiles));
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    SegPlan pl = workspace ? plan_segments(B * H, Tlen) : SegPlan{1, (Tlen + SB - 1) / SB};
-    if (pl.nseg > MAX_SEG) pl = SegPlan{1, (Tlen + SB - 1) / SB};
+    const int nsb = (Tlen + SB - 1) / SB;
+    const SegPlan pl = workspace ? plan_segments(B * H, Tlen) : SegPlan{1, nsb, 1, nsb};
     float *ckpt = (workspace && keep_ckpt) ? (float *)workspace : nullptr;
     float *part = workspace ? (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H)) : nullptr;
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v;
     dim3 block(NT_F);
     if (pl.nseg > 1) {
-        dim3 grid(B * H * (pl.nseg - 1));
+        const int pieces = (pl.nseg - 1) * pl.m;
+        dim3 grid(B * H * pieces);
         if (per_token)
-            hipLaunchKernelGGL((forward<true, true>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk,
-                               vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part, floor_decay);
+            hipLaunchKernelGGL((forward<true, true>), grid, block, FWD_PASS_LDS, s, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, rr, kk, vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part,
+                               floor_decay);
         else
-            hipLaunchKernelGGL((forward<false, true>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr,
-                               kk, vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part, floor_decay);
+            hipLaunchKernelGGL((forward<false, true>), grid, block, FWD_PASS_LDS, s, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, rr, kk, vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part,
+                               floor_decay);
+        hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, 0, pieces - 1, 1, pl.m,
+                           pl.nseg * pl.m, s_in, part);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(B * H * pl.nseg);
+    dim3 grid(B * H * pl.nseg), block16(NT_F16);
     prof_begin(KID_CHUNK_FORWARD, s);
     if (per_token)
-        hipLaunchKernelGGL((forward<true, false>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv,
-                           w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+        hipLaunchKernelGGL((forward16<true>), grid, block16, sizeof(Fwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
+                           vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
     else
-        hipLaunchKernelGGL((forward<false, false>), grid, block, sizeof(FwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk,
+        hipLaunchKernelGGL((forward16<false>), grid, block16, sizeof(Fwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
                            vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
     prof_end(KID_CHUNK_FORWARD, s);
     return hipGetLastError();
@@ -1047,33 +1795,49 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
     if (!attr_done) {
         hipError_t e = allow_lds(backward<true>, sizeof(BwdTiles));
         if (e == hipSuccess) e = allow_lds(backward<false>, sizeof(BwdTiles));
+        if (e == hipSuccess) e = allow_lds(backward16<true>, sizeof(Bwd16Tiles));
+        if (e == hipSuccess) e = allow_lds(backward16<false>, sizeof(Bwd16Tiles));
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    SegPlan pl = plan_segments(B * H, Tlen);
-    if (pl.nseg > MAX_SEG) pl = SegPlan{1, (Tlen + SB - 1) / SB};
+    const SegPlan pl = plan_segments(B * H, Tlen);
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v, *gg = (const bf16 *)gy;
     if (pl.nseg > 1) {
-        dim3 grid(B * H * (pl.nseg - 1)), block(NT_F);
+        const int pieces = (pl.nseg - 1) * pl.m;
+        dim3 grid(B * H * pieces), block(NT_F);
         if (per_token)
-            hipLaunchKernelGGL((gradient_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, rr, w, gg, gpart,
-                               floor_decay);
+            hipLaunchKernelGGL((gradient_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, w,
+                               gg, gpart, floor_decay);
         else
-            hipLaunchKernelGGL((gradient_pass<false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, rr, w, gg, gpart,
-                               floor_decay);
+            hipLaunchKernelGGL((gradient_pass<false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, w,
+                               gg, gpart, floor_decay);
+        hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, pl.nseg * pl.m - 1, pl.m,
+                           -1, pl.m, pl.nseg * pl.m, gs_out, gpart);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(B * H * pl.nseg), block(NT_B);
+    dim3 grid(B * H * pl.nseg), block(NT_B), block16(NT_B16);
+    static const bool old_kernel = getenv("RWKV_WKV_BWD8") != nullptr;
     prof_begin(KID_CHUNK_BACKWARD, s);
-    if (per_token)
-        hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv, w,
-                           u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in,
-                           floor_decay);
-    else
-        hipLaunchKernelGGL((backward<false>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, rr, kk, vv, w,
-                           u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr, gw_part,
-                           gu_part, gs_in, floor_decay);
+    if (old_kernel) {
+        if (per_token)
+            hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk, vv,
+                               w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in,
+                               floor_decay);
+        else
+            hipLaunchKernelGGL((backward<false>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk, vv,
+                               w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr, gw_part,
+                               gu_part, gs_in, floor_decay);
+    } else {
+        if (per_token)
+            hipLaunchKernelGGL((backward16<true>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr,
+                               kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part,
+                               gs_in, floor_decay);
+        else
+            hipLaunchKernelGGL((backward16<false>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr,
+                               kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr,
+                               gw_part, gu_part, gs_in, floor_decay);
+    }
     prof_end(KID_CHUNK_BACKWARD, s);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
