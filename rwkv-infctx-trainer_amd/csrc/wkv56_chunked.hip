@@ -48,6 +48,13 @@ namespace chunked {
 #define PT_PRINT(name)
 #endif
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load, which would stall each phase on the prefetch of the next step;
+// the wavefronts of these kernels talk to each other through LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 typedef short s4 __attribute__((ext_vector_type(4)));
 typedef short s8 __attribute__((ext_vector_type(8)));
 typedef __bf16 b8 __attribute__((ext_vector_type(8)));
@@ -306,7 +313,7 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
             }
         }
         PT_MARK(0)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(1)
         if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
 
@@ -341,7 +348,7 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
             split2(at[0], at[1], h0, l0);
             split2(at[2], at[3], h1, l1);
             sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
-            __syncthreads();
+            lds_barrier();
         }
 
         // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
@@ -388,7 +395,7 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
             }
         }
         PT_MARK(2)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(3)
     }
     PT_PRINT(STATE_ONLY ? "fwd-state" : "fwd")
@@ -419,21 +426,21 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
 }
 
 // ------------------------------------------------------- forward, 16 wavefronts --
-// The main forward pass with the work of a 64-token step spread over 16 wavefronts:
-// wavefront (q, wv) produces y for block q (16 tokens), value columns 16wv..16wv+15.
-// Every wavefront holds the state at the step's start and advances its own copy
-// over the q blocks before its own (a few MFMAs per block, far cheaper than the
-// block's own work); the wavefronts of the last block advance once more and hand the
-// state at the step's end to the others through LDS.  Four wavefronts per SIMD keep
-// the vector ALU busy where one wavefront alone cannot issue fast enough.
+// The main forward pass with the work of a 64-token step spread over 16 wavefronts
+// (four per SIMD).  A step runs in three phases separated by workgroup barriers:
 //
-// Staging: lane = (token of a block, four channels), a block's running log decay is
-// a prefix sum over the 16 lanes of a DPP row.  Every tile is [token][channel]; the
-// operands that the MFMAs want with the tokens along the contraction (k e^{b-incl}, v)
-// come out of the transposing LDS read of gfx950.
+//   prepare   all wavefronts: lane = (token of a block, four channels); a block's running
+//             log decay is a prefix sum over the 16 lanes of a DPP row.  Every tile is
+//             [token][channel]; the operands that the MFMAs want with the tokens along the
+//             contraction (k e^{b-incl}, v) come out of the transposing LDS read of gfx950.
+//   chains    wavefronts 0-7 own the state for good: wavefront (w, half) holds keys
+//             32*half..32*half+31 x values 16w..16w+15 in registers, walks it over the four
+//             blocks and leaves its share of  rh S  per block in LDS;
+//             wavefronts 8-11 build the masked intra-block matrix of one block each.
+//   finish    wavefront (q, w): y of block q, value columns 16w..16w+15 = the two shares
+//             + (intra-block matrix) v, converted and stored.
 constexpr int NT_F16 = 1024;
-constexpr int LDT = 80;       // row length of the tiles read through the transposing load: four rows of
-                              // eight dwords each must fall into distinct bank groups (40 dwords = 8 mod 32)
+constexpr int LDT = LD;       // tiles read through the transposing load use the same padded row length
 
 struct Fwd16Tiles {
     uint16_t rh[SB * LD];     // r e^{excl}       [token][key]  bf16 head / remainder
@@ -446,7 +453,7 @@ struct Fwd16Tiles {
     float dec[4][HEAD];       // e^{b} per block and key
     float rho[4][SB];         // r . (u o k) per token: partial sums over 16 channels each
     uint4 amat[4][64];        // masked intra-block matrix of each block as A-operand fragments (head, remainder)
-    float4 hand[4][4][64];    // state at the end of the step, accumulator layout [wv][kk][lane]
+    float4 yi[2][4][4][64];   // rh S per key half, block, value quarter: accumulator layout, one float4 per lane
 };
 
 __device__ __forceinline__ float row_prefix_sum(float x) {      // inclusive, over the 16 lanes of a DPP row
@@ -479,23 +486,24 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
     Fwd16Tiles &sm = *reinterpret_cast<Fwd16Tiles *>(smem_raw);
     const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
-    const int q = w16 >> 2, wv = w16 & 3;
+    const int q = w16 >> 2, wv = w16 & 3;          // block and quarter for preparing and finishing
+    const bool chain = w16 < 8, builder = w16 >= 8 && w16 < 12;
+    const int hk = w16 >> 2;                       // chain wavefronts: key half
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
     const int sb0 = seg * sps, sb1 = min(nsb, (seg + 1) * sps);
 
-    // state at the start of the step: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]
-    f4 S[4];
-    {
+    // chain wavefronts: S[j][e] = S[key 32hk+16j+4g+e][value 16wv+n]
+    f4 S[2] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
+    if (chain) {
         const float *sp = seg == 0 ? s_in + (size_t)bh * HEAD * HEAD : part + ((size_t)bh * nseg * m + seg * m - 1) * PART;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
+            for (int e = 0; e < 4; e++) S[j][e] = sp[(32 * hk + 16 * j + 4 * g + e) * HEAD + 16 * wv + n];
     }
-    // staging role: token n of block q, channels c4..c4+3
+    // preparing role: token n of block q, channels c4..c4+3
     const int c4 = 16 * wv + 4 * g, tok = 16 * q + n;
-    const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
@@ -518,6 +526,8 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
         }
     };
     const int tro = tr_lane_offset(lane, LDT);
+    // the slot of this wavefront's two state tiles in a checkpoint (accumulator layout)
+    const size_t ck_off = (size_t)bh * (nsb + 1) * HEAD * HEAD;
 
     fetch(sb0);
     PT_DECL
@@ -528,6 +538,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             float l[4] = {pw.x, pw.y, pw.z, pw.w}, inc[4], tot[4];
             const float rf[4] = {bf_lo(pr.x), bf_hi(pr.x), bf_lo(pr.y), bf_hi(pr.y)};
             const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
+            const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
             float rhv[4], knv[4], khv[4], p = 0.f;
 #pragma unroll
@@ -558,30 +569,44 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             if (g == 0) sm.rho[wv][tok] = p;
         }
         PT_MARK(0)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(1)
         if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
 
-        if (ckpt && q == 0) {       // state at the start of this step, 16 bytes per lane and tile
-            float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + sb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
-        }
-        // one block of the state recurrence: S <- e^{b} o S + (k e^{b-incl})^T v
-        auto advance = [&](int blk) {
-            const s4 v_op = frag_tr(sm.v, tro + (16 * blk) * LDT + 16 * wv);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][16 * kk + 4 * g]);
-                S[kk][0] *= d4.x; S[kk][1] *= d4.y; S[kk][2] *= d4.z; S[kk][3] *= d4.w;
-                S[kk] = mma2(frag_tr(sm.kh, tro + (16 * blk) * LDT + 16 * kk), frag_tr(sm.khl, tro + (16 * blk) * LDT + 16 * kk),
-                             v_op, v_op, S[kk]);
+        if (chain) {
+            if (ckpt) {       // state at the start of this step, 16 bytes per lane and tile
+                float4 *cp = reinterpret_cast<float4 *>(ckpt + ck_off + (size_t)sb * HEAD * HEAD) + (wv * 4 + 2 * hk) * 64 + lane;
+                cp[0] = make_float4(S[0][0], S[0][1], S[0][2], S[0][3]);
+                cp[64] = make_float4(S[1][0], S[1][1], S[1][2], S[1][3]);
             }
-        };
-        if (q == wv) {
-            // ---------------- builds the masked intra-block matrix of block q for the wavefronts (q, *):
+            // ---------------- the state over the four blocks; per block this half's share of rh S
+#pragma unroll
+            for (int blk = 0; blk < 4; blk++) {
+                const int row = 16 * blk + n, ca = 32 * hk + 4 * g, cb = ca + 16;
+                s4 s0h, s0l, s1h, s1l;
+                split4(S[0], s0h, s0l);
+                split4(S[1], s1h, s1l);
+                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                f4 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0;
+                y0 = mma2(r0, r1, s0h, s1h, y0);
+                y1 = mma2(r0, r1, s0l, s1l, y1);
+                y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
+                // S <- e^{b} o S + (k e^{b-incl})^T v
+                const s4 v_op = frag_tr(sm.v, tro + (16 * blk) * LDT + 16 * wv);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][32 * hk + 16 * j + 4 * g]);
+                    S[j][0] *= d4.x; S[j][1] *= d4.y; S[j][2] *= d4.z; S[j][3] *= d4.w;
+                    S[j] = mma2(frag_tr(sm.kh, tro + (16 * blk) * LDT + 32 * hk + 16 * j),
+                                frag_tr(sm.khl, tro + (16 * blk) * LDT + 32 * hk + 16 * j), v_op, v_op, S[j]);
+                }
+                y0 += y1 + y2;
+                sm.yi[hk][blk][wv][lane] = make_float4(y0[0], y0[1], y0[2], y0[3]);
+            }
+        } else if (builder) {
+            // ---------------- the masked intra-block matrix of block wv, once for everybody:
             // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n
-            const int row = 16 * q + n;
+            const int row = 16 * wv + n;
             f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
 #pragma unroll
             for (int kk = 0; kk < 4; kk += 2) {
@@ -602,32 +627,18 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             uint32_t h0, l0, h1, l1;                        // A[t = n][s = 4g..4g+3] as head + remainder
             split2(at[0], at[1], h0, l0);
             split2(at[2], at[3], h1, l1);
-            sm.amat[q][lane] = make_uint4(h0, h1, l0, l1);
+            sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
         }
-        // the state at the start of block q (wave-uniform trip count)
-        for (int blk = 0; blk < q; blk++) advance(blk);
         PT_MARK(2)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(3)
 
         // ---------------- y of block q, value columns 16wv..16wv+15
         if (y && sb * SB + 16 * q < Tlen) {
-            const int row = 16 * q + n;
-            f4 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                s4 s0h, s0l, s1h, s1l;
-                split4(S[kk], s0h, s0l);
-                split4(S[kk + 1], s1h, s1l);
-                y0 = mma2(r0, r1, s0h, s1h, y0);
-                y1 = mma2(r0, r1, s0l, s1l, y1);
-                y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
-            }
+            const float4 ya = sm.yi[0][q][wv][lane], yb = sm.yi[1][q][wv][lane];
             const uint4 am = sm.amat[q][lane];
             const s4 v_op = frag_tr(sm.v, tro + (16 * q) * LDT + 16 * wv);
-            f4 yt = y0 + (y1 + y2);
+            f4 yt = {ya.x + yb.x, ya.y + yb.y, ya.z + yb.z, ya.w + yb.w};
             yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
             bf16 *yp = y + base + (size_t)(sb * SB + 16 * q + 4 * g) * C + 16 * wv + n;
             const int left = Tlen - (sb * SB + 16 * q + 4 * g);
@@ -635,34 +646,22 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             for (int e = 0; e < 4; e++)
                 if (e < left) yp[(size_t)e * C] = bf16{bf16_bits(yt[e])};
         }
-        if (q == 3) {         // on to the end of the step, for everybody
-            advance(3);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) sm.hand[wv][kk][lane] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
-        }
         PT_MARK(4)
-        __syncthreads();
-        if (q != 3) {
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                const float4 x = sm.hand[wv][kk][lane];
-                S[kk] = f4{x.x, x.y, x.z, x.w};
-            }
-        }
+        lds_barrier();
     }
     PT_PRINT("fwd16")
-    if (seg == nseg - 1 && q == 3) {
+    if (chain && seg == nseg - 1) {
         if (ckpt) {       // the final state takes the slot after the last step
-            float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + nsb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+            float4 *cp = reinterpret_cast<float4 *>(ckpt + ck_off + (size_t)nsb * HEAD * HEAD) + (wv * 4 + 2 * hk) * 64 + lane;
+            cp[0] = make_float4(S[0][0], S[0][1], S[0][2], S[0][3]);
+            cp[64] = make_float4(S[1][0], S[1][1], S[1][2], S[1][3]);
         }
         if (s_out) {
             float *op = s_out + (size_t)bh * HEAD * HEAD;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++)
+            for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int e = 0; e < 4; e++) op[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
+                for (int e = 0; e < 4; e++) op[(32 * hk + 16 * j + 4 * g + e) * HEAD + 16 * wv + n] = S[j][e];
         }
     }
 }
@@ -845,7 +844,7 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
             if ((lane & 3) == 0) sm.rho[chh][tk0 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1)] = tot_p;
         }
         PT_MARK(0)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(1)
         if (sb > sb0) fetch(sb - 1);
 
@@ -1048,7 +1047,7 @@ __global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nse
             }
         }
         PT_MARK(2)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(3)
     }
     PT_PRINT("bwd")
@@ -1156,7 +1155,7 @@ __global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, in
             gg_.put(sm.gyT, ot);
             if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(ra + oa), __expf(rb + ob));
         }
-        __syncthreads();
+        lds_barrier();
         if (sb > sb0) fetch(sb - 1);
 #pragma unroll
         for (int q = 3; q >= 0; q--) {
@@ -1171,7 +1170,7 @@ __global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, in
                              gyTf, gyTf, G[kk]);
             }
         }
-        __syncthreads();
+        lds_barrier();
     }
     float *pp = gpart + ((size_t)bh * nseg * m + piece) * PART;
 #pragma unroll
@@ -1377,7 +1376,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         }
       }
         PT_MARK(0)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(1)
 
         f4 KG[4];                    // wavefronts 8-11: kh G per block, KG[q][e] at [token 4g+e][value own]
@@ -1522,7 +1521,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         }
       }
         PT_MARK(2)
-        __syncthreads();
+        lds_barrier();
         PT_MARK(3)
 
         float Dloc[4], lfac[4];
@@ -1592,7 +1591,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         }
       }
         PT_MARK(4)
-        __syncthreads();
+        lds_barrier();
         {
             WKV_LOCAL_LANE
             float A_end = sm.arun[own];          // at the end of block q: the step's end plus the later blocks
@@ -1609,7 +1608,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
         if (role == 0 && g == 0) sm.arun[own] += (sm.tots[0][own] + sm.tots[1][own]) + (sm.tots[2][own] + sm.tots[3][own]);
     }
 
@@ -1626,7 +1625,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         sm.red[0][q][own] = gu_acc;
         sm.red[1][q][own] = gw_acc;
     }
-    __syncthreads();
+    lds_barrier();
     if (q == 0 && g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
         const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
         gu_part[po] = (sm.red[0][0][own] + sm.red[0][1][own]) + (sm.red[0][2][own] + sm.red[0][3][own]);
