@@ -451,9 +451,10 @@ struct Fwd16Tiles {
     uint16_t khl[SB * LDT];
     uint16_t v[SB * LDT];     // v                [token][value] (read transposed)
     float dec[4][HEAD];       // e^{b} per block and key
-    float rho[4][SB];         // r . (u o k) per token: partial sums over 16 channels each
+    float rho[SB];            // r . (u o k) per token
     uint4 amat[4][64];        // masked intra-block matrix of each block as A-operand fragments (head, remainder)
     float4 yi[2][4][4][64];   // rh S per key half, block, value quarter: accumulator layout, one float4 per lane
+    float wtot[16][HEAD];     // per wavefront (four tokens) and channel: sum of log w, for the block-wide running sum
 };
 
 __device__ __forceinline__ float row_prefix_sum(float x) {      // inclusive, over the 16 lanes of a DPP row
@@ -473,6 +474,44 @@ __device__ __forceinline__ int tr_lane_offset(int lane, int ld) {
 __device__ __forceinline__ s4 frag_tr(const uint16_t *tile, int off) {
     typedef s4 __attribute__((address_space(3))) lds_s4;
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)(tile + off));
+}
+
+// Preparing role of the 16-wavefront kernels: a lane holds one token and four channels;
+// the 16 lanes of a DPP row are the 64 channels of that token (one 128-byte row of the
+// (B,T,C) bf16 tensors, so every global access is a full row segment); wavefront w has the
+// tokens 4w..4w+3 of the step, four wavefronts make a 16-token block.
+// block_scan: from log w of the lane's token to the inclusive running sum inside the
+// block (inc) and the block total (tot).  Inside a wavefront two shuffles; across the four
+// wavefronts of a block through `wtot` in LDS (one workgroup barrier, executed by all).
+__device__ __forceinline__ void block_scan(const float (&l)[4], float (&inc)[4], float (&tot)[4], float (*wtot)[HEAD],
+                                           int w16, int g, int n) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        float x = l[c];
+        const float u1 = __shfl_up(x, 16);
+        x += g >= 1 ? u1 : 0.f;
+        const float u2 = __shfl_up(x, 32);
+        x += g >= 2 ? u2 : 0.f;
+        inc[c] = x;
+    }
+    if (g == 3) *reinterpret_cast<float4 *>(&wtot[w16][4 * n]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
+    lds_barrier();
+    const int w0 = w16 & ~3, pos = w16 & 3;
+    float pre[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 4; c++) tot[c] = 0.f;
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+        const float4 t4 = *reinterpret_cast<const float4 *>(&wtot[w0 + x][4 * n]);
+        const float tv[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            tot[c] += tv[c];
+            pre[c] += x < pos ? tv[c] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++) inc[c] += pre[c];
 }
 
 template <bool PER_TOKEN_W>
@@ -502,8 +541,9 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
 #pragma unroll
             for (int e = 0; e < 4; e++) S[j][e] = sp[(32 * hk + 16 * j + 4 * g + e) * HEAD + 16 * wv + n];
     }
-    // preparing role: token n of block q, channels c4..c4+3
-    const int c4 = 16 * wv + 4 * g, tok = 16 * q + n;
+    // preparing role: token tok of the step (block q), channels c4..c4+3
+    const int c4 = 4 * n, tok = 4 * w16 + g;
+    const bool last_tok = (w16 & 3) == 3 && g == 3;        // the block's last token
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
@@ -529,6 +569,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
     // the slot of this wavefront's two state tiles in a checkpoint (accumulator layout)
     const size_t ck_off = (size_t)bh * (nsb + 1) * HEAD * HEAD;
 
+    bool have_y = false;
     fetch(sb0);
     PT_DECL
     for (int sb = sb0; sb < sb1; sb++) {
@@ -540,15 +581,21 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
             const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
+            if (PER_TOKEN_W) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) l[c] = log_decay(l[c], floor_decay);
+            }
+            if (have_y) {      // y of the previous step waits in the rh tile: out as full rows, by the lanes that overwrite it next
+                const int t = (sb - 1) * SB + tok;
+                if (t < Tlen) *reinterpret_cast<uint2 *>(y + base + (size_t)t * C + c4) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
+            }
+            block_scan(l, inc, tot, sm.wtot, w16, g, n);
             float rhv[4], knv[4], khv[4], p = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                if (PER_TOKEN_W) l[c] = log_decay(l[c], floor_decay);
-                inc[c] = row_prefix_sum(l[c]);
-                tot[c] = __shfl(inc[c], lane | 15);
                 rhv[c] = rf[c] * __expf(inc[c] - l[c]);
                 khv[c] = kf[c] * __expf(tot[c] - inc[c]);
-                knv[c] = n == 15 ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
+                knv[c] = last_tok ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
                 p = fmaf(rf[c] * uf[c], kf[c], p);
             }
             uint32_t h0, l0, h1, l1;
@@ -563,10 +610,9 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             *reinterpret_cast<uint2 *>(&sm.kh[ot]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.khl[ot]) = make_uint2(l0, l1);
             *reinterpret_cast<uint2 *>(&sm.v[ot]) = pv;
-            if (n == 15) *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
-            p += __shfl_xor(p, 16);
-            p += __shfl_xor(p, 32);
-            if (g == 0) sm.rho[wv][tok] = p;
+            if (last_tok) *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+            p = row_prefix_sum(p);           // lane 15 of the row ends with the sum over the 64 channels
+            if (n == 15) sm.rho[tok] = p;
         }
         PT_MARK(0)
         lds_barrier();
@@ -618,7 +664,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
                 a2 = mma2(k0, k1, frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), a2);
             }
             f4 at = a0 + (a1 + a2);
-            const float rho_t = (sm.rho[0][row] + sm.rho[1][row]) + (sm.rho[2][row] + sm.rho[3][row]);
+            const float rho_t = sm.rho[row];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int s_ = 4 * g + e;
@@ -634,20 +680,23 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
         PT_MARK(3)
 
         // ---------------- y of block q, value columns 16wv..16wv+15
-        if (y && sb * SB + 16 * q < Tlen) {
+        if (y) {
             const float4 ya = sm.yi[0][q][wv][lane], yb = sm.yi[1][q][wv][lane];
             const uint4 am = sm.amat[q][lane];
             const s4 v_op = frag_tr(sm.v, tro + (16 * q) * LDT + 16 * wv);
             f4 yt = {ya.x + yb.x, ya.y + yb.y, ya.z + yb.z, ya.w + yb.w};
             yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
-            bf16 *yp = y + base + (size_t)(sb * SB + 16 * q + 4 * g) * C + 16 * wv + n;
-            const int left = Tlen - (sb * SB + 16 * q + 4 * g);
+            // into the rh tile (nobody reads it any more in this step), [token][value]; it leaves as full rows
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (e < left) yp[(size_t)e * C] = bf16{bf16_bits(yt[e])};
+            for (int e = 0; e < 4; e++) sm.rh[(16 * q + 4 * g + e) * LD + 16 * wv + n] = bf16_bits(yt[e]);
         }
         PT_MARK(4)
         lds_barrier();
+        have_y = y != nullptr;
+    }
+    if (have_y) {
+        const int t = (sb1 - 1) * SB + tok;
+        if (t < Tlen) *reinterpret_cast<uint2 *>(y + base + (size_t)t * C + c4) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
     }
     PT_PRINT("fwd16")
     if (chain && seg == nseg - 1) {
@@ -1218,7 +1267,8 @@ struct Bwd16Tiles {
     float lw[SB * HEAD];     // log w                                         [token][key]
     float tot[4][HEAD];      // b per block and key
     float dec[4][HEAD];      // e^{b}
-    float rho[4][SB];        // r . (u o k) per token: partial sums over 16 channels each
+    float rho[SB];           // r . (u o k) per token
+    float wtot[16][HEAD];    // per wavefront (four tokens) and channel: sum of log w, for the block-wide running sum
     float q1[SB * HEAD];     // gy S^T          [token][key]
     float q4[SB * HEAD];     // v G^T           [token][key]
     uint4 pfr[4][2][64];     // per block: P^T masked to s < t, P masked to t > s, as A-operand fragments (head, remainder)
@@ -1235,8 +1285,8 @@ constexpr int NT_B16 = 1024;
 #define WKV_LOCAL_LANE                                                                                        \
     int lane_v_ = lane0;                                                                                      \
     asm volatile("" : "+v"(lane_v_));                                                                         \
-    const int lane = lane_v_, g = lane >> 4, n = lane & 15, own = 16 * wv + n, c4 = 16 * wv + 4 * g,           \
-              tok = 16 * q + n, tro = tr_lane_offset(lane, LD);                                               \
+    const int lane = lane_v_, g = lane >> 4, n = lane & 15, own = 16 * wv + n, c4 = 4 * n,                     \
+              tok = 4 * w16 + g, tro = tr_lane_offset(lane, LD);                                              \
     (void)tro; (void)c4; (void)tok; (void)own;
 
 template <bool PER_TOKEN_W>
@@ -1292,8 +1342,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
     }
     float gu_acc = 0.f, gw_acc = 0.f;
 
-    // preparing role: token n of block q, channels c4..c4+3
-    const int c4 = 16 * wv + 4 * g, tok = 16 * q + n;
+    // preparing role: token tok of the step (block q), channels c4..c4+3 (one 128-byte row per 16 lanes)
+    const int c4 = 4 * n, tok = 4 * w16 + g;
+    const bool last_tok = (w16 & 3) == 3 && g == 3;        // the block's last token
+    bool have_out = false;
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
@@ -1317,6 +1369,18 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         }
     };
     const int lane0 = lane;
+    // gr, gk, gv (and gw) of a finished step wait in the rh, kh, v tiles (and the incl table), [token][channel];
+    // they leave as full rows, written by the lanes that overwrite those entries next
+    auto write_out = [&](int sb, int tok, int c4) {
+        const int t = sb * SB + tok;
+        if (t < Tlen) {
+            const size_t o = base + (size_t)t * C + c4;
+            *reinterpret_cast<uint2 *>(gr + o) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
+            *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
+            *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
+            if (PER_TOKEN_W) *reinterpret_cast<float4 *>(gw_tok + o) = *reinterpret_cast<const float4 *>(&sm.incl[tok * HEAD + c4]);
+        }
+    };
 
     fetch(sb1 - 1, tok, c4);
     PT_DECL
@@ -1340,15 +1404,18 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
             const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
+            if (PER_TOKEN_W) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) l[c] = log_decay(l[c], floor_decay);
+            }
+            if (have_out) write_out(sb + 1, tok, c4);
+            block_scan(l, inc, tot, sm.wtot, w16, g, n);
             float rhv[4], knv[4], khv[4], p = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                if (PER_TOKEN_W) l[c] = log_decay(l[c], floor_decay);
-                inc[c] = row_prefix_sum(l[c]);
-                tot[c] = __shfl(inc[c], lane | 15);
                 rhv[c] = rf[c] * __expf(inc[c] - l[c]);
                 khv[c] = kf[c] * __expf(tot[c] - inc[c]);
-                knv[c] = n == 15 ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
+                knv[c] = last_tok ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
                 p = fmaf(rf[c] * uf[c], kf[c], p);
             }
             uint32_t h0, l0, h1, l1;
@@ -1366,13 +1433,12 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             *reinterpret_cast<uint2 *>(&sm.khl[o]) = make_uint2(l0, l1);
             *reinterpret_cast<float4 *>(&sm.incl[tok * HEAD + c4]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
             *reinterpret_cast<float4 *>(&sm.lw[tok * HEAD + c4]) = make_float4(l[0], l[1], l[2], l[3]);
-            if (n == 15) {
+            if (last_tok) {
                 *reinterpret_cast<float4 *>(&sm.tot[q][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
                 *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
             }
-            p += __shfl_xor(p, 16);
-            p += __shfl_xor(p, 32);
-            if (g == 0) sm.rho[wv][tok] = p;
+            p = row_prefix_sum(p);           // lane 15 of the row ends with the sum over the 64 channels
+            if (n == 15) sm.rho[tok] = p;
         }
       }
         PT_MARK(0)
@@ -1509,7 +1575,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 a2 = mma2(r0, r1, frag(sm.knl, row, ca), frag(sm.knl, row, cb), a2);
             }
             f4 at = a0 + (a1 + a2);
-            const float rho_s = (sm.rho[0][row] + sm.rho[1][row]) + (sm.rho[2][row] + sm.rho[3][row]);
+            const float rho_s = sm.rho[row];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int x = 4 * g + e;
@@ -1534,11 +1600,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 const uint4 am = sm.amat[qq][lane];
                 const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
                 const f4 gvt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), gyTf, gyTf, KG[qq]);
-                bf16 *gp = gv + base + (size_t)(sb * SB + 16 * qq + 4 * g) * C + own;
-                const int left = Tlen - (sb * SB + 16 * qq + 4 * g);
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (e < left) gp[(size_t)e * C] = bf16{bf16_bits(gvt[e])};
+                for (int e = 0; e < 4; e++) sm.v[(16 * qq + 4 * g + e) * LD + own] = bf16_bits(gvt[e]);      // v is not read any more
             }
         }
         // ---------------- block q, keys 16wv..16wv+15: gr, gk, decay gradient
@@ -1558,7 +1621,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int tk = 16 * q + 4 * g + e;
-                const int t = sb * SB + tk;
                 const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
                 const float E1 = __expf(exc), E2 = __expf(tot_i - inc);
                 const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
@@ -1572,11 +1634,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 z[e] = kr * gkn;
                 lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
                 gu_acc = fmaf(rr * kr, pd, gu_acc);
-                if (t < Tlen) {
-                    const size_t o = base + (size_t)t * C;
-                    gr[o + own] = bf16{bf16_bits(grv)};
-                    gk[o + own] = bf16{bf16_bits(gkv)};
-                }
+                // this wavefront was the only reader left of its (block, quarter) corner of the rh and kh tiles
+                sm.rh[tk * LD + own] = bf16_bits(grv);
+                sm.kh[tk * LD + own] = bf16_bits(gkv);
             }
             // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over the block's later tokens of c
             const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
@@ -1602,7 +1662,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 const int t = sb * SB + 16 * q + 4 * g + e;
                 const float Dt = A_end + Dloc[e];
                 if (PER_TOKEN_W) {
-                    if (t < Tlen) gw_tok[base + (size_t)t * C + own] = Dt * lfac[e];
+                    sm.incl[(16 * q + 4 * g + e) * HEAD + own] = Dt * lfac[e];
                 } else {
                     gw_acc += (t < Tlen) ? Dt : 0.f;
                 }
@@ -1610,7 +1670,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         }
         lds_barrier();
         if (role == 0 && g == 0) sm.arun[own] += (sm.tots[0][own] + sm.tots[1][own]) + (sm.tots[2][own] + sm.tots[3][own]);
+        have_out = true;
     }
+    if (have_out) write_out(sb0, tok, c4);
 
     PT_PRINT("bwd16")
     if (role == 1 && gs_in && seg == 0) {
