@@ -22,16 +22,22 @@
 // two 16-deep products per 16x16x32 instruction.  This is what keeps the decay
 // gradient, a difference of large running sums, at fp32-like accuracy.
 //
-// The scaled operands are prepared 64 tokens at a time (a lane keeps the running
-// log decay of its tokens in registers; one or two shuffles join the pieces of a
-// block) and laid out in LDS so that every MFMA operand fragment is one 8-byte
-// read; rows are padded to 68 elements, which spreads the 16 rows of a fragment
-// over all banks.
+// The scaled operands are prepared 64 tokens at a time and laid out in LDS as
+// [token][channel] tiles whose rows are padded to 68 elements, which makes every 8-byte
+// MFMA operand fragment read conflict-free, both the plain ones (tokens along M or N)
+// and the transposing ones (tokens along the contraction).
+//
+// The main kernels run 16 wavefronts per workgroup, four per SIMD: one wavefront alone
+// issues a vector instruction only every six to eight cycles, so the work of a step is
+// cut into independent pieces (per 16-token block, per 16 channels) for different
+// wavefronts, and only the short serial recurrences stay with one wavefront each.
+// Global memory is always touched in full 128-byte rows (16 lanes x 8 bytes = the 64
+// channels of one token and head).
 //
 // Time-parallel split: a sequence is cut into segments that run as separate
-// workgroups; a light pass leaves each segment's effect on a state handed in
-// (S_out = decay o S_in + delta), the main pass folds the earlier segments'
-// summaries in order.  Backward does the same with the state gradient.
+// workgroups; a light pass leaves each piece's effect on a state handed in
+// (S_out = decay o S_in + delta), a small kernel chains the summaries into the state
+// at the start of every segment.  Backward does the same with the state gradient.
 #include "common.h"
 
 namespace wkv {
@@ -62,8 +68,7 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 constexpr int SB = 64;        // tokens prepared per staging step
 constexpr int LD = 68;        // padded row length of a 64x64 bf16 tile in LDS
-constexpr int NT_F = 256;     // forward: 4 wavefronts
-constexpr int NT_B = 512;     // backward: 8 wavefronts (4 key-side + 4 value-side)
+constexpr int NT_F = 256;     // summary passes: 4 wavefronts
 
 // One 16-deep product, D[m][n] += sum_k A[m][k] B[k][n].  Issued as a 16x16x32 MFMA
 // with a zero upper half: on gfx950 a 16x16x16 MFMA chained on the accumulator of a
@@ -108,44 +113,6 @@ __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane g
     return x;
 }
 
-// sum each of 8 per-lane values over the 32 lanes of a half wavefront; afterwards
-// lane L holds the total of value index 4*b4 + 2*b3 + b2 (bK = bit K of L)
-__device__ __forceinline__ float sum8_over_half(const float (&p)[8], int lane) {
-    float a4[4], a2[2];
-    const bool h4 = lane & 16, h3 = lane & 8, h2 = lane & 4;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        const float keep = h4 ? p[e + 4] : p[e], send = h4 ? p[e] : p[e + 4];
-        a4[e] = keep + __shfl_xor(send, 16);
-    }
-#pragma unroll
-    for (int e = 0; e < 2; e++) {
-        const float keep = h3 ? a4[e + 2] : a4[e], send = h3 ? a4[e] : a4[e + 2];
-        a2[e] = keep + __shfl_xor(send, 8);
-    }
-    const float keep = h2 ? a2[1] : a2[0], send = h2 ? a2[0] : a2[1];
-    float x = keep + __shfl_xor(send, 4);
-    x += __shfl_xor(x, 2);
-    x += __shfl_xor(x, 1);
-    return x;
-}
-__device__ __forceinline__ int sum8_index(int lane) { return ((lane >> 4) & 1) * 4 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1); }
-// the same for 4 values over 16 lanes: lane L ends with the total of index 2*b3 + b2
-__device__ __forceinline__ float sum4_over_16(const float (&p)[4], int lane) {
-    float a2[2];
-    const bool h3 = lane & 8, h2 = lane & 4;
-#pragma unroll
-    for (int e = 0; e < 2; e++) {
-        const float keep = h3 ? p[e + 2] : p[e], send = h3 ? p[e] : p[e + 2];
-        a2[e] = keep + __shfl_xor(send, 8);
-    }
-    const float keep = h2 ? a2[1] : a2[0], send = h2 ? a2[0] : a2[1];
-    float x = keep + __shfl_xor(send, 4);
-    x += __shfl_xor(x, 2);
-    x += __shfl_xor(x, 1);
-    return x;
-}
-
 // collects N tokens of a channel pair (one packed pair per token) into two rows of a [channel][token] tile
 template <int N>
 struct Gather {
@@ -168,76 +135,48 @@ struct Gather {
 // handed back (backward).  [key][value] fp32 plus one decay per key.
 constexpr int PART = HEAD * HEAD + HEAD;
 
-// ------------------------------------------------------------------- forward --
-struct FwdTiles {
-    // the summary pass uses (and allocates) only the part up to `rh`
+// -------------------------------------------------------------- summary passes --
+// Time-parallel split.  One piece (`pps` steps) of the segments 0..nseg-2, from a zero
+// state: what the piece does to a state handed in, S_out = decay o S_in + delta.
+// fold_summaries then chains the pieces into the state at the start of every segment.
+// Four wavefronts; wavefront w owns value columns 16w..16w+15 of the state; a lane
+// prepares eight tokens of a channel pair (running log decay in registers, one
+// shuffle joins the two halves of a block).
+struct StatePassTiles {
     uint16_t khT[SB * LD];   // k e^{b-incl}     [key][token]   bf16 head of the value
     uint16_t khTl[SB * LD];  //                                 bf16 remainder
     uint16_t vT[SB * LD];    // v                [value][token]
     float dec[4][HEAD];      // e^{b} per block and key
-    uint16_t rh[SB * LD];    // r e^{excl}       [token][key]
-    uint16_t rhl[SB * LD];
-    uint16_t kn[SB * LD];    // k e^{-incl}      [token][key]
-    uint16_t knl[SB * LD];
-    float rho[SB];           // r . (u o k) per token
-    uint4 amat[4][64];       // the masked intra-block matrix of each block as MFMA A-operand fragments
-                             // (head, remainder), one 16-byte entry per lane; built once, used by all wavefronts
 };
-constexpr size_t FWD_PASS_LDS = offsetof(FwdTiles, rh);
 
-// Forward over one segment (`sps` 64-token steps) of one (batch, head); grid =
-// B*H*nseg, 4 wavefronts; wavefront w owns value columns 16w..16w+15 of the state.
-//   STATE_ONLY pass  (segments 0..nseg-2, each cut into `m` pieces of `pps` steps so
-//                    that the pass itself fills the GPU): from a zero state, leaves the
-//                    piece's summary in `part`; fold_forward then turns the summaries
-//                    into the state at the start of every segment;
-//   main pass        (all segments): starts from that state (segment 0: from s_in)
-//                    and produces y.
-// ckpt (optional) receives the state at the start of every 64-token step and, in one more slot, the final state, fp32, in the
-// accumulator layout of this kernel: [bh][step][value/16][key/16][lane][4] with
-// lane = 16*((key%16)/4) + value%16 and the last index = key%4; the last segment writes s_out.
-template <bool PER_TOKEN_W, bool STATE_ONLY>
-__global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
-        const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
-        const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
-        bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, float *__restrict__ part,
-        int floor_decay)
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(NT_F) void state_pass(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
+        const bf16 *__restrict__ k, const bf16 *__restrict__ v, const float *__restrict__ wraw,
+        float *__restrict__ part, int floor_decay)
 {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    FwdTiles &sm = *reinterpret_cast<FwdTiles *>(smem_raw);
-    const int units = STATE_ONLY ? (nseg - 1) * m : nseg;       // workgroups per (batch, head)
-    const int bh = blockIdx.x / units, unit = blockIdx.x % units, b = bh / H, h = bh % H;
-    const int seg = STATE_ONLY ? unit / m : unit;
+    __shared__ __align__(16) StatePassTiles sm;
+    const int units = (nseg - 1) * m;       // workgroups per (batch, head)
+    const int bh = blockIdx.x / units, unit = blockIdx.x % units, b = bh / H, h = bh % H, seg = unit / m;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = STATE_ONLY ? seg * sps + (unit % m) * pps : seg * sps;
-    const int sb1 = min(min(nsb, (seg + 1) * sps), STATE_ONLY ? sb0 + pps : nsb);
+    const int sb0 = seg * sps + (unit % m) * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
 
-    // state tiles: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]
+    // state tiles: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]; Dacc = product of the decays
     f4 S[4], Dacc[4];
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
         S[kk] = f4{0.f, 0.f, 0.f, 0.f};
         Dacc[kk] = f4{1.f, 1.f, 1.f, 1.f};
     }
-    if (!STATE_ONLY) {       // segment 0 starts from s_in, a later one from what fold_forward left
-        const float *sp = seg == 0 ? s_in + (size_t)bh * HEAD * HEAD : part + ((size_t)bh * nseg * m + seg * m - 1) * PART;
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) S[kk][e] = sp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n];
-    }
-    // staging role: block wv of the step, tokens 8*half..8*half+7 of it, channels c0, c0+1
+    // preparing role: block wv of the step, tokens 8*half..8*half+7 of it, channels c0, c0+1
     const int half = lane >> 5, c0 = 2 * (lane & 31);
-    const float2 u_c = *reinterpret_cast<const float2 *>(u + h * HEAD + c0);
     float2 l_const = make_float2(0.f, 0.f);
     if (!PER_TOKEN_W) {
         l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
         l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
     }
-
-    uint32_t pr[8], pk[8], pv[8];
+    uint32_t pk[8], pv[8];
     float2 pw[8];
     auto fetch = [&](int sb) {
 #pragma unroll
@@ -245,59 +184,35 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
             const int t = sb * SB + 16 * wv + 8 * half + x;
             if (t < Tlen) {
                 const size_t o = base + (size_t)t * C + c0;
-                if (!STATE_ONLY) pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
                 pk[x] = *reinterpret_cast<const uint32_t *>(k + o);
                 pv[x] = *reinterpret_cast<const uint32_t *>(v + o);
                 pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
             } else {
-                pr[x] = pk[x] = pv[x] = 0;
+                pk[x] = pv[x] = 0;
                 pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);   // log w = 0
             }
         }
     };
-
-    fetch(sb0);
-    PT_DECL
+    if (sb0 < sb1) fetch(sb0);
     for (int sb = sb0; sb < sb1; sb++) {
-        PT_MARK(4)
-        // ---------------- prepare the scaled operands of 64 tokens
         {
-            float ia[8], ib[8], la[8], lb[8];
+            float ia[8], ib[8];
             float ra = 0.f, rb = 0.f;
 #pragma unroll
             for (int x = 0; x < 8; x++) {
-                la[x] = PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
-                lb[x] = PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
-                ra += la[x]; rb += lb[x];
+                ra += PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
+                rb += PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
                 ia[x] = ra; ib[x] = rb;
             }
             // the other half of the block sits in lane ^ 32
             const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
             const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
             const float tota = ra + oa, totb = rb + ob;
-            const float enta = __expf(-tota), entb = __expf(-totb);
-            float p[8];
             Gather<8> gk_h, gk_l, gv_;
 #pragma unroll
             for (int x = 0; x < 8; x++) {
-                const float inca = ia[x] + offa, incb = ib[x] + offb;
-                const float kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
-                const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
-                const int o = (16 * wv + 8 * half + x) * LD + c0;
                 uint32_t hi, lo;
-                if (!STATE_ONLY) {
-                    const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]);
-                    split2(rfa * __expf(inca - la[x]), rfb * __expf(incb - lb[x]), hi, lo);
-                    *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
-                    *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
-                    // k e^{-incl}; the block's last token has no later token and is never used
-                    const bool last = half && x == 7;
-                    split2(last ? 0.f : kha * enta, last ? 0.f : khb * entb, hi, lo);
-                    *reinterpret_cast<uint32_t *>(&sm.kn[o]) = hi;
-                    *reinterpret_cast<uint32_t *>(&sm.knl[o]) = lo;
-                    p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
-                }
-                split2(kha, khb, hi, lo);
+                split2(bf_lo(pk[x]) * __expf(tota - (ia[x] + offa)), bf_hi(pk[x]) * __expf(totb - (ib[x] + offb)), hi, lo);
                 gk_h.add(x, hi);
                 gk_l.add(x, lo);
                 gv_.add(x, pv[x]);
@@ -307,122 +222,32 @@ __global__ __launch_bounds__(NT_F) void forward(int Tlen, int C, int H, int nseg
             gk_l.put(sm.khTl, ot);
             gv_.put(sm.vT, ot);
             if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(tota), __expf(totb));
-            if (!STATE_ONLY) {
-                const float tot_p = sum8_over_half(p, lane);
-                if ((lane & 3) == 0) sm.rho[16 * wv + 8 * half + sum8_index(lane)] = tot_p;
-            }
         }
-        PT_MARK(0)
         lds_barrier();
-        PT_MARK(1)
         if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
-
-        if (!STATE_ONLY) {
-            if (ckpt) {       // state at the start of this step, 16 bytes per lane and tile
-                float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + sb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
-            }
-            // ---------------- wavefront q builds the masked intra-block matrix of block q for everybody:
-            // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n.  Three independent
-            // accumulators (head*head, rem*head, head*rem) shorten the dependency chain.
-            const int row = 16 * wv + n;
-            f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
-                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                a0 = mma2(k0, k1, r0, r1, a0);
-                a1 = mma2(frag(sm.knl, row, ca), frag(sm.knl, row, cb), r0, r1, a1);
-                a2 = mma2(k0, k1, frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), a2);
-            }
-            f4 at = a0 + (a1 + a2);
-            const float rho_t = sm.rho[16 * wv + n];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int s_ = 4 * g + e;
-                at[e] = s_ < n ? at[e] : (s_ == n ? rho_t : 0.f);
-            }
-            uint32_t h0, l0, h1, l1;                        // A[t = n][s = 4g..4g+3] as head + remainder
-            split2(at[0], at[1], h0, l0);
-            split2(at[2], at[3], h1, l1);
-            sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
-            lds_barrier();
-        }
-
-        // ---------------- four 16-token blocks; this wavefront: value columns 16wv..16wv+15
-        const bool full = (sb + 1) * SB <= Tlen;
-        bf16 *ystep = y + base + (size_t)(sb * SB) * C;
-        const unsigned ylane = (unsigned)(4 * g) * C + 16 * wv + n;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            if (sb * SB + 16 * q >= Tlen) break;
-            const int row = 16 * q + n;
             const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
-            if (!STATE_ONLY) {
-                // inter-block part of y: rh S, with S as head + remainder
-                f4 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0;
-#pragma unroll
-                for (int kk = 0; kk < 4; kk += 2) {
-                    const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                    const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                    s4 s0h, s0l, s1h, s1l;
-                    split4(S[kk], s0h, s0l);
-                    split4(S[kk + 1], s1h, s1l);
-                    y0 = mma2(r0, r1, s0h, s1h, y0);
-                    y1 = mma2(r0, r1, s0l, s1l, y1);
-                    y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
-                }
-                const uint4 am = sm.amat[q][lane];
-                f4 yt = y0 + (y1 + y2);
-                yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
-                if (y) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const unsigned o = ylane + (unsigned)(16 * q + e) * C;
-                        if (full || sb * SB + 16 * q + 4 * g + e < Tlen) ystep[o] = bf16{bf16_bits(yt[e])};
-                    }
-                }
-            }
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) {
                 const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
                 S[kk][0] *= d4.x; S[kk][1] *= d4.y; S[kk][2] *= d4.z; S[kk][3] *= d4.w;
-                if (STATE_ONLY) { Dacc[kk][0] *= d4.x; Dacc[kk][1] *= d4.y; Dacc[kk][2] *= d4.z; Dacc[kk][3] *= d4.w; }
+                Dacc[kk][0] *= d4.x; Dacc[kk][1] *= d4.y; Dacc[kk][2] *= d4.z; Dacc[kk][3] *= d4.w;
                 S[kk] = mma2(frag(sm.khT, 16 * kk + n, 16 * q + 4 * g), frag(sm.khTl, 16 * kk + n, 16 * q + 4 * g),
                              v_op, v_op, S[kk]);
             }
         }
-        PT_MARK(2)
         lds_barrier();
-        PT_MARK(3)
     }
-    PT_PRINT(STATE_ONLY ? "fwd-state" : "fwd")
-    if (STATE_ONLY) {
-        float *pp = part + ((size_t)bh * nseg * m + unit) * PART;
+    float *pp = part + ((size_t)bh * nseg * m + unit) * PART;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++)
+    for (int kk = 0; kk < 4; kk++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int row = 16 * kk + 4 * g + e;
-                pp[row * HEAD + 16 * wv + n] = S[kk][e];
-                if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
-            }
-    } else if (seg == nseg - 1) {
-        if (ckpt) {       // the final state takes the slot after the last step
-            float4 *cp = reinterpret_cast<float4 *>(ckpt + ((size_t)bh * (nsb + 1) + nsb) * HEAD * HEAD) + (wv * 4) * 64 + lane;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) cp[kk * 64] = make_float4(S[kk][0], S[kk][1], S[kk][2], S[kk][3]);
+        for (int e = 0; e < 4; e++) {
+            const int row = 16 * kk + 4 * g + e;
+            pp[row * HEAD + 16 * wv + n] = S[kk][e];
+            if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
         }
-        if (s_out) {
-            float *op = s_out + (size_t)bh * HEAD * HEAD;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) op[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = S[kk][e];
-        }
-    }
 }
 
 // ------------------------------------------------------- forward, 16 wavefronts --
@@ -716,412 +541,6 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
 }
 
 // ------------------------------------------------------------------ backward --
-// Walks the 64-token steps of a segment from the last to the first.  Per step:
-// prepare the operands, rebuild the state at the start of each of its four blocks
-// from the step's checkpoint, then take the blocks in reverse.  With G the gradient
-// of the state at a block's end, P[t][s] = gy_t . v_s, rh = r e^{excl}, kh = k e^{b-incl}:
-//
-//   gr_t = e^{excl_t} (gy_t S^T) + e^{excl_t-b} sum_{s<t} P[t][s] kh_s + u k_t P[t][t]
-//   gk_s = e^{-incl_s} sum_{t>s} P[t][s] rh_t + e^{b-incl_s} (v_s G^T) + u r_s P[s][s]
-//   gv_s = sum_{t>=s} A~[t][s] gy_t + kh_s G          (A~ = the forward's masked matrix)
-//   G   <- e^{b} o G + rh^T gy
-//
-// and the decay gradient from the running sum  A_{t-1} = A_t + r_t gr_t - k_t gk_t,
-// dL/dlog w_t = A_t - k_t (gk_t - u r_t P[t][t]),  re-anchored at every step end
-// to sum_j G o S.
-//
-// Eight wavefronts: all of them prepare the operands; then wavefronts 0-3 ("key
-// side", key channels 16w..16w+15) rebuild the state and produce gr, gk, gw, gu with
-// G held value-major, while wavefronts 4-7 ("value side", value channels 16w..16w+15)
-// produce gv with a second, key-major copy of G.  Neither side needs anything the
-// other computes, so two wavefronts per SIMD hide each other's latencies.
-struct BwdTiles {
-    uint16_t gy[SB * LD];    // gy              [token][value]
-    uint16_t v[SB * LD];     // v               [token][value]
-    uint16_t rh[SB * LD];    // r e^{excl}      [token][key]   head / remainder
-    uint16_t rhl[SB * LD];
-    uint16_t kn[SB * LD];    // k e^{-incl}     [token][key]
-    uint16_t knl[SB * LD];
-    uint16_t kh[SB * LD];    // k e^{b-incl}    [token][key]
-    uint16_t khl[SB * LD];
-    uint16_t gyT[SB * LD];   // gy              [value][token]
-    uint16_t vT[SB * LD];    // v               [value][token]
-    uint16_t khT[SB * LD];   // k e^{b-incl}    [key][token]
-    uint16_t khTl[SB * LD];
-    uint16_t rhT[SB * LD];   // r e^{excl}      [key][token]
-    uint16_t rhTl[SB * LD];
-    float incl[SB * HEAD];   // inclusive running log decay inside the block [token][key]
-    float lw[SB * HEAD];     // log w                                         [token][key]
-    float tot[4][HEAD];      // b per block and key
-    float dec[4][HEAD];      // e^{b}
-    float rho[2][SB];        // r . (u o k) per token, one partial sum per half of the channels
-};
-
-template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_B) void backward(int Tlen, int C, int H, int nseg, int sps, int m,
-        const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
-        const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
-        const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
-        bf16 *__restrict__ gr, bf16 *__restrict__ gk, bf16 *__restrict__ gv, float *__restrict__ gw_tok,
-        float *__restrict__ gw_part, float *__restrict__ gu_part, float *__restrict__ gs_in, int floor_decay)
-{
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    BwdTiles &sm = *reinterpret_cast<BwdTiles *>(smem_raw);
-    const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
-    const int tid = threadIdx.x, w8 = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
-    const bool key_side = w8 < 4;
-    const int wv = w8 & 3;
-    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
-    const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = seg * sps, sb1 = min(nsb, sb0 + sps);
-    const int own = 16 * wv + n;                 // key channel (key side) / value channel (value side) of this lane
-    const float u_i = u[h * HEAD + own];
-
-    // key side:   G[kk][e] = G[key own][value 16kk+4g+e]
-    // value side: G[kk][e] = G[key 16kk+4g+e][value own]
-    f4 G[4];
-    {
-        // the last segment starts from gs_out, an earlier one from what fold_backward left
-        const float *gp = seg == nseg - 1 ? (gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr)
-                                          : gpart + ((size_t)bh * nseg * m + (seg + 1) * m) * PART;
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int x = 16 * kk + 4 * g + e;
-                G[kk][e] = gp ? (key_side ? gp[own * HEAD + x] : gp[x * HEAD + own]) : 0.f;
-            }
-    }
-    float A_run = 0.f, gu_acc = 0.f, gw_acc = 0.f;
-
-    // staging role: block sq of the step, tokens 8*half + 4*quarter .. +3 of it, channels c0, c0+1
-    const int sq = w8 >> 1, half = lane >> 5, quarter = (lane >> 4) & 1;
-    const int chh = w8 & 1, c0 = 2 * (16 * chh + (lane & 15));
-    const int tk0 = 16 * sq + 8 * half + 4 * quarter;
-    const float2 u_c = *reinterpret_cast<const float2 *>(u + h * HEAD + c0);
-    float2 l_const = make_float2(0.f, 0.f);
-    if (!PER_TOKEN_W) {
-        l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
-        l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
-    }
-    uint32_t pr[4], pk[4], pv[4], pg[4];
-    float2 pw[4];
-    auto fetch = [&](int sb) {
-#pragma unroll
-        for (int x = 0; x < 4; x++) {
-            const int t = sb * SB + tk0 + x;
-            if (t < Tlen) {
-                const size_t o = base + (size_t)t * C + c0;
-                pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
-                pk[x] = *reinterpret_cast<const uint32_t *>(k + o);
-                pv[x] = *reinterpret_cast<const uint32_t *>(v + o);
-                pg[x] = *reinterpret_cast<const uint32_t *>(gy + o);
-                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
-            } else {
-                pr[x] = pk[x] = pv[x] = pg[x] = 0;
-                pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);
-            }
-        }
-    };
-
-    fetch(sb1 - 1);
-    PT_DECL
-    for (int sb = sb1 - 1; sb >= sb0; sb--) {
-        PT_MARK(4)
-        // ---------------- prepare the operands of 64 tokens (all 8 wavefronts)
-        {
-            float ia[4], ib[4], la[4], lb[4];
-            float ra = 0.f, rb = 0.f;
-#pragma unroll
-            for (int x = 0; x < 4; x++) {
-                la[x] = PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
-                lb[x] = PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
-                ra += la[x]; rb += lb[x];
-                ia[x] = ra; ib[x] = rb;
-            }
-            // the block's four quarters sit in lanes ^16 and ^32
-            const float qa = __shfl_xor(ra, 16), qb = __shfl_xor(rb, 16);
-            const float pa = ra + qa, pb = rb + qb;                  // this half's 8 tokens
-            const float ha = __shfl_xor(pa, 32), hb = __shfl_xor(pb, 32);
-            const float tota = pa + ha, totb = pb + hb;
-            const float offa = (quarter ? qa : 0.f) + (half ? ha : 0.f), offb = (quarter ? qb : 0.f) + (half ? hb : 0.f);
-            const float enta = __expf(-tota), entb = __expf(-totb);
-            float p[4];
-            Gather<4> gk_h, gk_l, gr_h, gr_l, gv_, gg_;
-#pragma unroll
-            for (int x = 0; x < 4; x++) {
-                const float inca = ia[x] + offa, incb = ib[x] + offb;
-                const float rfa = bf_lo(pr[x]), rfb = bf_hi(pr[x]), kfa = bf_lo(pk[x]), kfb = bf_hi(pk[x]);
-                const float kha = kfa * __expf(tota - inca), khb = kfb * __expf(totb - incb);
-                const int tk = tk0 + x;
-                const int o = tk * LD + c0;
-                uint32_t hi, lo;
-                *reinterpret_cast<uint32_t *>(&sm.gy[o]) = pg[x];
-                *reinterpret_cast<uint32_t *>(&sm.v[o]) = pv[x];
-                split2(rfa * __expf(inca - la[x]), rfb * __expf(incb - lb[x]), hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.rh[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.rhl[o]) = lo;
-                gr_h.add(x, hi);
-                gr_l.add(x, lo);
-                const bool last = half && quarter && x == 3;       // no later token in the block: never used
-                split2(last ? 0.f : kha * enta, last ? 0.f : khb * entb, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.kn[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.knl[o]) = lo;
-                split2(kha, khb, hi, lo);
-                *reinterpret_cast<uint32_t *>(&sm.kh[o]) = hi;
-                *reinterpret_cast<uint32_t *>(&sm.khl[o]) = lo;
-                gk_h.add(x, hi);
-                gk_l.add(x, lo);
-                gv_.add(x, pv[x]);
-                gg_.add(x, pg[x]);
-                *reinterpret_cast<float2 *>(&sm.incl[tk * HEAD + c0]) = make_float2(inca, incb);
-                *reinterpret_cast<float2 *>(&sm.lw[tk * HEAD + c0]) = make_float2(la[x], lb[x]);
-                p[x] = rfa * u_c.x * kfa + rfb * u_c.y * kfb;
-            }
-            const int ot = c0 * LD + tk0;
-            gk_h.put(sm.khT, ot);
-            gk_l.put(sm.khTl, ot);
-            gr_h.put(sm.rhT, ot);
-            gr_l.put(sm.rhTl, ot);
-            gv_.put(sm.vT, ot);
-            gg_.put(sm.gyT, ot);
-            if (!half && !quarter) {
-                *reinterpret_cast<float2 *>(&sm.tot[sq][c0]) = make_float2(tota, totb);
-                *reinterpret_cast<float2 *>(&sm.dec[sq][c0]) = make_float2(__expf(tota), __expf(totb));
-            }
-            const float tot_p = sum4_over_16(p, lane);
-            if ((lane & 3) == 0) sm.rho[chh][tk0 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1)] = tot_p;
-        }
-        PT_MARK(0)
-        lds_barrier();
-        PT_MARK(1)
-        if (sb > sb0) fetch(sb - 1);
-
-        if (key_side) {
-            // ---------------- rebuild the state at the start of each block: ST[kk][e] = S[key own][value 16kk+4g+e]
-            f4 ST[4];
-            {   // checkpoint in the forward kernel's accumulator layout: element [key][value] sits at
-                // tile (value/16, key/16), lane 16*((key%16)/4) + value%16, component key%4
-                const float *cp = ckpt + ((size_t)bh * (nsb + 1) + sb) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) ST[kk][e] = cp[kk * 1024 + e * 4];
-            }
-            f4 Q1[4];                        // gy S^T per block, taken while S passes by: Q1[q][e] at [token 4g+e][key own]
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                Q1[q] = f4{0.f, 0.f, 0.f, 0.f};
-                if (sb * SB + 16 * q >= Tlen) continue;
-                {
-                    s4 sh[4], sl[4];
-#pragma unroll
-                    for (int kk = 0; kk < 4; kk++) split4(ST[kk], sh[kk], sl[kk]);
-                    f4 qa = {0.f, 0.f, 0.f, 0.f}, qb = qa;
-#pragma unroll
-                    for (int kk = 0; kk < 4; kk += 2) {
-                        const s4 y0 = frag(sm.gy, 16 * q + n, 16 * kk + 4 * g), y1 = frag(sm.gy, 16 * q + n, 16 * kk + 16 + 4 * g);
-                        qa = mma2(y0, y1, sh[kk], sh[kk + 1], qa);
-                        qb = mma2(y0, y1, sl[kk], sl[kk + 1], qb);
-                    }
-                    Q1[q] = qa + qb;
-                }
-                const float dq = sm.dec[q][own];
-                const s4 khf = frag(sm.khT, own, 16 * q + 4 * g), khfl = frag(sm.khTl, own, 16 * q + 4 * g);
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) {
-                    ST[kk] = ST[kk] * dq;
-                    const s4 vf_ = frag(sm.vT, 16 * kk + n, 16 * q + 4 * g);
-                    ST[kk] = mma2(vf_, vf_, khf, khfl, ST[kk]);
-                }
-            }
-            {   // anchor of the decay-gradient sum at the end of this step: sum_j G o S
-                float a = 0.f;
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) a = fmaf(G[kk][e], ST[kk][e], a);
-                A_run = group_sum4(a);
-            }
-            PT_MARK(5)
-            // ---------------- the four blocks, last first: gr, gk, gw, gu
-#pragma unroll
-            for (int q = 3; q >= 0; q--) {
-                if (sb * SB + 16 * q >= Tlen) continue;
-                const int row = 16 * q + n;
-                s4 gyf[4], vf[4];
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) {
-                    gyf[kk] = frag(sm.gy, row, 16 * kk + 4 * g);
-                    vf[kk] = frag(sm.v, row, 16 * kk + 4 * g);
-                }
-                // pt[e] = P[t = 4g+e][s = n],  ptT[e] = P[t = n][s = 4g+e]
-                f4 pt = {0.f, 0.f, 0.f, 0.f}, ptT = pt;
-                pt = mma2(gyf[0], gyf[1], vf[0], vf[1], pt);
-                ptT = mma2(vf[0], vf[1], gyf[0], gyf[1], ptT);
-                pt = mma2(gyf[2], gyf[3], vf[2], vf[3], pt);
-                ptT = mma2(vf[2], vf[3], gyf[2], gyf[3], ptT);
-                // state-gradient part while P is in flight: q4 = v G^T
-                f4 q1 = Q1[q], q4 = {0.f, 0.f, 0.f, 0.f}, q4b = q4;
-#pragma unroll
-                for (int kk = 0; kk < 4; kk += 2) {
-                    s4 g0h, g0l, g1h, g1l;
-                    split4(G[kk], g0h, g0l);
-                    split4(G[kk + 1], g1h, g1l);
-                    q4 = mma2(vf[kk], vf[kk + 1], g0h, g1h, q4);
-                    q4b = mma2(vf[kk], vf[kk + 1], g0l, g1l, q4b);
-                }
-                float pd[4];                                   // P[t][t] for this lane's tokens t = 4g+e
-                f4 pm, pTm;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    pd[e] = __shfl(pt[e], (lane & 48) | (4 * g + e));
-                    pm[e] = (4 * g + e > n) ? pt[e] : 0.f;     // later tokens t > s
-                    pTm[e] = (4 * g + e < n) ? ptT[e] : 0.f;   // earlier tokens s < t
-                }
-                s4 pm_h, pm_l, pT_h, pT_l;
-                split4(pm, pm_h, pm_l);
-                split4(pTm, pT_h, pT_l);
-                const s4 khTf = frag(sm.khT, own, 16 * q + 4 * g);     // kh[s = 4g..][key own]
-                const s4 khTfl = frag(sm.khTl, own, 16 * q + 4 * g);
-                const s4 rhTf = frag(sm.rhT, own, 16 * q + 4 * g);     // rh[t = 4g..][key own]
-                const s4 rhTfl = frag(sm.rhTl, own, 16 * q + 4 * g);
-                f4 q2 = {0.f, 0.f, 0.f, 0.f}, q2b = q2, q3 = q2, q3b = q2;
-                q2 = mma2(pT_h, pT_l, khTf, khTf, q2);
-                q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);
-                q2b = mma(pT_h, khTfl, q2b);
-                q3b = mma(pm_h, rhTfl, q3b);
-                q4 += q4b; q2 += q2b; q3 += q3b;
-
-                const float tot_i = sm.tot[q][own], ent_i = __expf(-tot_i);
-                float c[4], z[4], lfac[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int tk = 16 * q + 4 * g + e;
-                    const int t = sb * SB + tk;
-                    const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
-                    const float E1 = __expf(exc), E2 = __expf(tot_i - inc);
-                    // r, k back from their scaled head + remainder (16 mantissa bits)
-                    const float rr = (bf2f(sm.rh[tk * LD + own]) + bf2f(sm.rhl[tk * LD + own])) * __expf(-exc);
-                    const float kr = (bf2f(sm.kh[tk * LD + own]) + bf2f(sm.khl[tk * LD + own])) * __expf(inc - tot_i);
-                    const float grv = E1 * (q1[e] + ent_i * q2[e]) + u_i * kr * pd[e];
-                    const float gkn = E2 * (ent_i * q3[e] + q4[e]);
-                    const float gkv = gkn + u_i * rr * pd[e];
-                    c[e] = rr * grv - kr * gkv;
-                    z[e] = kr * gkn;
-                    lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
-                    gu_acc = fmaf(rr * kr, pd[e], gu_acc);
-                    if (t < Tlen) {
-                        const size_t o = base + (size_t)t * C;
-                        gr[o + own] = bf16{bf16_bits(grv)};
-                        gk[o + own] = bf16{bf16_bits(gkv)};
-                    }
-                }
-                {   // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over later tokens of c
-                    const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
-                    const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
-                    const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
-                    const float all = group_sum4(mine);
-                    const float suf[4] = {suf0, suf1, suf2, 0.f};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const float Dt = A_run + later + suf[e] - z[e];
-                        const int t = sb * SB + 16 * q + 4 * g + e;
-                        if (PER_TOKEN_W) {
-                            if (t < Tlen) gw_tok[base + (size_t)t * C + own] = Dt * lfac[e];
-                        } else {
-                            gw_acc += (t < Tlen) ? Dt : 0.f;
-                        }
-                    }
-                    A_run += all;
-                }
-                {   // G <- e^{b} o G + rh^T gy  (value-major copy: one decay per lane)
-                    const float dq = sm.dec[q][own];
-#pragma unroll
-                    for (int kk = 0; kk < 4; kk++) {
-                        G[kk] = G[kk] * dq;
-                        const s4 gT_ = frag(sm.gyT, 16 * kk + n, 16 * q + 4 * g);
-                        G[kk] = mma2(gT_, gT_, rhTf, rhTfl, G[kk]);
-                    }
-                }
-            }
-        } else {
-            // ---------------- value side: gv for value channel `own`, key-major G
-#pragma unroll
-            for (int q = 3; q >= 0; q--) {
-                if (sb * SB + 16 * q >= Tlen) continue;
-                const int row = 16 * q + n;
-                // the forward's masked matrix: at[e] = A~[t = 4g+e][s = n], three independent accumulators;
-                // and kh G with G as head + remainder
-                f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, g0 = a0, g1 = a0, g2 = a0;
-#pragma unroll
-                for (int kk = 0; kk < 4; kk += 2) {
-                    const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                    const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                    const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
-                    a0 = mma2(r0, r1, k0, k1, a0);
-                    a1 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), k0, k1, a1);
-                    a2 = mma2(r0, r1, frag(sm.knl, row, ca), frag(sm.knl, row, cb), a2);
-                    s4 g0h, g0l, g1h, g1l;
-                    split4(G[kk], g0h, g0l);
-                    split4(G[kk + 1], g1h, g1l);
-                    const s4 h0 = frag(sm.kh, row, ca), h1 = frag(sm.kh, row, cb);
-                    g0 = mma2(h0, h1, g0h, g1h, g0);
-                    g1 = mma2(h0, h1, g0l, g1l, g1);
-                    g2 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g2);
-                }
-                f4 at = a0 + (a1 + a2);
-                {
-                    const float rho_s = sm.rho[0][16 * q + n] + sm.rho[1][16 * q + n];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) at[e] = (4 * g + e > n) ? at[e] : ((4 * g + e == n) ? rho_s : 0.f);
-                }
-                s4 a_h, a_l;
-                split4(at, a_h, a_l);
-                const s4 gyTf = frag(sm.gyT, own, 16 * q + 4 * g);     // gy[t = 4g..][value own]
-                f4 gvt = g0 + (g1 + g2);
-                gvt = mma2(a_h, a_l, gyTf, gyTf, gvt);                 // gv[s = 4g+e][value own]
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int t = sb * SB + 16 * q + 4 * g + e;
-                    if (t < Tlen) gv[base + (size_t)t * C + own] = bf16{bf16_bits(gvt[e])};
-                }
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) {   // G <- e^{b} o G + rh^T gy  (key-major copy: one decay per row)
-                    const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
-                    G[kk][0] *= d4.x; G[kk][1] *= d4.y; G[kk][2] *= d4.z; G[kk][3] *= d4.w;
-                    G[kk] = mma2(frag(sm.rhT, 16 * kk + n, 16 * q + 4 * g), frag(sm.rhTl, 16 * kk + n, 16 * q + 4 * g),
-                                 gyTf, gyTf, G[kk]);
-                }
-            }
-        }
-        PT_MARK(2)
-        lds_barrier();
-        PT_MARK(3)
-    }
-    PT_PRINT("bwd")
-
-    if (key_side) {
-        if (gs_in && seg == 0) {
-            float *gp = gs_in + (size_t)bh * HEAD * HEAD + own * HEAD;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++)
-                *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(G[kk][0], G[kk][1], G[kk][2], G[kk][3]);
-        }
-        gu_acc = group_sum4(gu_acc);
-        gw_acc = group_sum4(gw_acc);
-        if (g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
-            const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
-            gu_part[po] = gu_acc;
-            if (!PER_TOKEN_W) {
-                bool fl;
-                const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
-                gw_part[po] = fl ? 0.f : gw_acc * l;
-            }
-        }
-    }
-}
-
 // State-gradient summary of one piece (`pps` steps) of the segments 1..nseg-1 for the
 // backward split: from a zero gradient, walks the piece's tokens last to first with
 //   G <- e^{b} o G + (r e^{excl})^T gy      per 16-token block
@@ -1233,13 +652,25 @@ __global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, in
 }
 
 // ------------------------------------------------------ backward, 16 wavefronts --
-// The same mathematics as `backward`, with the work of a 64-token step spread over 16
-// wavefronts (four per SIMD) so that no single wavefront's instruction stream is the
-// critical path.  A step runs in three phases separated by workgroup barriers:
+// Walks the 64-token steps of a segment from the last to the first.  With S the state
+// at a block's start, G the gradient of the state at a block's end, P[t][s] = gy_t . v_s,
+// rh = r e^{excl}, kh = k e^{b-incl}:
 //
-//   prepare   all wavefronts: lane = (token of a block, four channels), every tile is
-//             [token][channel]; fragments with the tokens along the contraction come
-//             from the transposing LDS read.
+//   gr_t = e^{excl_t} (gy_t S^T) + e^{excl_t-b} sum_{s<t} P[t][s] kh_s + u k_t P[t][t]
+//   gk_s = e^{-incl_s} sum_{t>s} P[t][s] rh_t + e^{b-incl_s} (v_s G^T) + u r_s P[s][s]
+//   gv_s = sum_{t>=s} A~[t][s] gy_t + kh_s G          (A~ = the forward's masked matrix)
+//   G   <- e^{b} o G + rh^T gy
+//
+// and the decay gradient from the running sum  A_{t-1} = A_t + r_t gr_t - k_t gk_t,
+// dL/dlog w_t = A_t - k_t (gk_t - u r_t P[t][t]).
+//
+// The work of a step is spread over 16 wavefronts (four per SIMD) so that no single
+// wavefront's instruction stream is the critical path.  A step runs in three phases
+// separated by workgroup barriers:
+//
+//   prepare   all wavefronts: lane = (one token, four channels), 16 lanes = one 128-byte
+//             row of the inputs; every tile is [token][channel]; fragments with the tokens
+//             along the contraction come from the transposing LDS read.
 //   chains    wavefronts  0-3  walk the state forward from the step's checkpoint and
 //                              leave  Q1 = gy S^T  of each block in LDS;
 //             wavefronts  4-7  walk the state gradient backward (value-major copy) and
@@ -1250,10 +681,13 @@ __global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, in
 //   blocks    wavefront (q, w): gr, gk and the decay gradient of block q, keys
 //             16w..16w+15; wavefronts 8-11 also finish gv.
 //
+// Results go back into LDS tiles that are no longer read ([token][channel]) and leave
+// as full rows at the start of the next step, written by the lanes that overwrite them.
+//
 // The running sum of the decay gradient is anchored once per segment (at the segment's
-// end, from the state checkpoint there and the gradient handed in) and carried from
-// step to step in LDS; inside a step every block sums its own tokens and the blocks
-// are joined through LDS.
+// end, from the state checkpoint there and the gradient handed in: sum_j G o S) and
+// carried from step to step in LDS; inside a step every block sums its own tokens and
+// the blocks are joined through LDS.
 struct Bwd16Tiles {
     uint16_t gy[SB * LD];    // gy              [token][value]
     uint16_t v[SB * LD];     // v               [token][value]
@@ -1815,12 +1249,10 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
         const int pieces = (pl.nseg - 1) * pl.m;
         dim3 grid(B * H * pieces);
         if (per_token)
-            hipLaunchKernelGGL((forward<true, true>), grid, block, FWD_PASS_LDS, s, Tlen, C, H, pl.nseg, pl.sps, pl.m,
-                               pl.pps, rr, kk, vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part,
+            hipLaunchKernelGGL((state_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w, part,
                                floor_decay);
         else
-            hipLaunchKernelGGL((forward<false, true>), grid, block, FWD_PASS_LDS, s, Tlen, C, H, pl.nseg, pl.sps, pl.m,
-                               pl.pps, rr, kk, vv, w, u, s_in, (bf16 *)nullptr, (float *)nullptr, (float *)nullptr, part,
+            hipLaunchKernelGGL((state_pass<false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w, part,
                                floor_decay);
         hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, 0, pieces - 1, 1, pl.m,
                            pl.nseg * pl.m, s_in, part);
@@ -1854,9 +1286,7 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
     }
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = allow_lds(backward<true>, sizeof(BwdTiles));
-        if (e == hipSuccess) e = allow_lds(backward<false>, sizeof(BwdTiles));
-        if (e == hipSuccess) e = allow_lds(backward16<true>, sizeof(Bwd16Tiles));
+        hipError_t e = allow_lds(backward16<true>, sizeof(Bwd16Tiles));
         if (e == hipSuccess) e = allow_lds(backward16<false>, sizeof(Bwd16Tiles));
         if (e != hipSuccess) return e;
         attr_done = true;
@@ -1877,28 +1307,16 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(B * H * pl.nseg), block(NT_B), block16(NT_B16);
-    static const bool old_kernel = getenv("RWKV_WKV_BWD8") != nullptr;
+    dim3 grid(B * H * pl.nseg), block16(NT_B16);
     prof_begin(KID_CHUNK_BACKWARD, s);
-    if (old_kernel) {
-        if (per_token)
-            hipLaunchKernelGGL((backward<true>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk, vv,
-                               w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in,
-                               floor_decay);
-        else
-            hipLaunchKernelGGL((backward<false>), grid, block, sizeof(BwdTiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk, vv,
-                               w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr, gw_part,
-                               gu_part, gs_in, floor_decay);
-    } else {
-        if (per_token)
-            hipLaunchKernelGGL((backward16<true>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr,
-                               kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part,
-                               gs_in, floor_decay);
-        else
-            hipLaunchKernelGGL((backward16<false>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr,
-                               kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr,
-                               gw_part, gu_part, gs_in, floor_decay);
-    }
+    if (per_token)
+        hipLaunchKernelGGL((backward16<true>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
+                           vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in,
+                           floor_decay);
+    else
+        hipLaunchKernelGGL((backward16<false>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
+                           vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr, gw_part,
+                           gu_part, gs_in, floor_decay);
     prof_end(KID_CHUNK_BACKWARD, s);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
