@@ -107,6 +107,21 @@ __device__ __forceinline__ void split4(f4 x, s4 &hi, s4 &lo) {
     hi = as_s4(h0, h1);
     lo = as_s4(l0, l1);
 }
+// The builders' r operand of the masked intra-block matrix: (r e^{excl}) e^{-b} = r e^{excl-b}, from the head/remainder
+// fragments of r e^{excl} (four keys of one token) and e^{-b} of those keys, as head + remainder again.  With
+// k e^{b-incl} as the other operand the product is r k e^{excl_t - incl_s}, at most |r k| where it is used (s < t).
+// A block's first token has no earlier token; its row is zeroed (its exponent -b is the only one beyond 79.5).
+__device__ __forceinline__ void scale_split(s4 hi, s4 lo, float4 f, bool zero, s4 &oh, s4 &ol) {
+    const uint2 h = __builtin_bit_cast(uint2, hi), l = __builtin_bit_cast(uint2, lo);
+    float x0 = (bf_lo(h.x) + bf_lo(l.x)) * f.x, x1 = (bf_hi(h.x) + bf_hi(l.x)) * f.y;
+    float x2 = (bf_lo(h.y) + bf_lo(l.y)) * f.z, x3 = (bf_hi(h.y) + bf_hi(l.y)) * f.w;
+    if (zero) x0 = x1 = x2 = x3 = 0.f;
+    uint32_t h0, l0, h1, l1;
+    split2(x0, x1, h0, l0);
+    split2(x2, x3, h1, l1);
+    oh = as_s4(h0, h1);
+    ol = as_s4(l0, l1);
+}
 __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane groups of 16
     x += __shfl_xor(x, 16);
     x += __shfl_xor(x, 32);
@@ -270,12 +285,11 @@ constexpr int LDT = LD;       // tiles read through the transposing load use the
 struct Fwd16Tiles {
     uint16_t rh[SB * LD];     // r e^{excl}       [token][key]  bf16 head / remainder
     uint16_t rhl[SB * LD];
-    uint16_t kn[SB * LD];     // k e^{-incl}      [token][key]
-    uint16_t knl[SB * LD];
-    uint16_t kh[SB * LDT];    // k e^{b-incl}     [token][key]   (read transposed)
+    uint16_t kh[SB * LDT];    // k e^{b-incl}     [token][key]   (read both ways)
     uint16_t khl[SB * LDT];
     uint16_t v[SB * LDT];     // v                [token][value] (read transposed)
     float dec[4][HEAD];       // e^{b} per block and key
+    float ent[4][HEAD];       // e^{-b}
     float rho[SB];            // r . (u o k) per token
     uint4 amat[4][64];        // masked intra-block matrix of each block as A-operand fragments (head, remainder)
     float4 yi[2][4][4][64];   // rh S per key half, block, value quarter: accumulator layout, one float4 per lane
@@ -305,11 +319,13 @@ __device__ __forceinline__ s4 frag_tr(const uint16_t *tile, int off) {
 // the 16 lanes of a DPP row are the 64 channels of that token (one 128-byte row of the
 // (B,T,C) bf16 tensors, so every global access is a full row segment); wavefront w has the
 // tokens 4w..4w+3 of the step, four wavefronts make a 16-token block.
-// block_scan: from log w of the lane's token to the inclusive running sum inside the
-// block (inc) and the block total (tot).  Inside a wavefront two shuffles; across the four
-// wavefronts of a block through `wtot` in LDS (one workgroup barrier, executed by all).
-__device__ __forceinline__ void block_scan(const float (&l)[4], float (&inc)[4], float (&tot)[4], float (*wtot)[HEAD],
-                                           int w16, int g, int n) {
+// Block-wide running sum of log w in two halves, so that the exchange across the four wavefronts of a block
+// rides on a barrier the step has anyway:
+//   scan_local  (at the end of the previous step, on the prefetched w): log w of the lane's token -> running sum
+//               inside the wavefront (two shuffles); the wavefront's total goes to `wtot` in LDS;
+//   scan_join   (at the start of the step, after that barrier): adds the totals of the earlier wavefronts of the
+//               block (inc = inclusive running sum inside the block) and forms the block total (tot).
+__device__ __forceinline__ void scan_local(const float (&l)[4], float (&inc)[4], float (*wtot)[HEAD], int w16, int g, int n) {
 #pragma unroll
     for (int c = 0; c < 4; c++) {
         float x = l[c];
@@ -320,23 +336,17 @@ __device__ __forceinline__ void block_scan(const float (&l)[4], float (&inc)[4],
         inc[c] = x;
     }
     if (g == 3) *reinterpret_cast<float4 *>(&wtot[w16][4 * n]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
-    lds_barrier();
-    const int w0 = w16 & ~3, pos = w16 & 3;
-    float pre[4] = {0.f, 0.f, 0.f, 0.f};
+}
+__device__ __forceinline__ void scan_join(float (&inc)[4], float (&tot)[4], const float (*wtot)[HEAD], int w16, int n) {
+    const int w0 = w16 & ~3, pos = w16 & 3;       // wavefront-uniform
 #pragma unroll
     for (int c = 0; c < 4; c++) tot[c] = 0.f;
 #pragma unroll
     for (int x = 0; x < 4; x++) {
         const float4 t4 = *reinterpret_cast<const float4 *>(&wtot[w0 + x][4 * n]);
-        const float tv[4] = {t4.x, t4.y, t4.z, t4.w};
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            tot[c] += tv[c];
-            pre[c] += x < pos ? tv[c] : 0.f;
-        }
+        tot[0] += t4.x; tot[1] += t4.y; tot[2] += t4.z; tot[3] += t4.w;
+        if (x < pos) { inc[0] += t4.x; inc[1] += t4.y; inc[2] += t4.z; inc[3] += t4.w; }
     }
-#pragma unroll
-    for (int c = 0; c < 4; c++) inc[c] += pre[c];
 }
 
 template <bool PER_TOKEN_W>
@@ -368,7 +378,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
     }
     // preparing role: token tok of the step (block q), channels c4..c4+3
     const int c4 = 4 * n, tok = 4 * w16 + g;
-    const bool last_tok = (w16 & 3) == 3 && g == 3;        // the block's last token
+
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
@@ -396,31 +406,38 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
 
     bool have_y = false;
     fetch(sb0);
+    // log w of this lane's token and its running sum inside the wavefront, always one step ahead (see scan_local)
+    float lc[4], ic[4];
+    auto scan_ahead = [&]() {
+        lc[0] = pw.x; lc[1] = pw.y; lc[2] = pw.z; lc[3] = pw.w;
+        if (PER_TOKEN_W) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) lc[c] = log_decay(lc[c], floor_decay);
+        }
+        scan_local(lc, ic, sm.wtot, w16, g, n);
+    };
+    scan_ahead();
+    lds_barrier();
     PT_DECL
     for (int sb = sb0; sb < sb1; sb++) {
         PT_MARK(5)
         // ---------------- prepare the scaled operands of this lane's token
         {
-            float l[4] = {pw.x, pw.y, pw.z, pw.w}, inc[4], tot[4];
+            float l[4] = {lc[0], lc[1], lc[2], lc[3]}, inc[4] = {ic[0], ic[1], ic[2], ic[3]}, tot[4];
             const float rf[4] = {bf_lo(pr.x), bf_hi(pr.x), bf_lo(pr.y), bf_hi(pr.y)};
             const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
             const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
-            if (PER_TOKEN_W) {
-#pragma unroll
-                for (int c = 0; c < 4; c++) l[c] = log_decay(l[c], floor_decay);
-            }
             if (have_y) {      // y of the previous step waits in the rh tile: out as full rows, by the lanes that overwrite it next
                 const int t = (sb - 1) * SB + tok;
                 if (t < Tlen) *reinterpret_cast<uint2 *>(y + base + (size_t)t * C + c4) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
             }
-            block_scan(l, inc, tot, sm.wtot, w16, g, n);
-            float rhv[4], knv[4], khv[4], p = 0.f;
+            scan_join(inc, tot, sm.wtot, w16, n);
+            float rhv[4], khv[4], p = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 rhv[c] = rf[c] * __expf(inc[c] - l[c]);
                 khv[c] = kf[c] * __expf(tot[c] - inc[c]);
-                knv[c] = last_tok ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
                 p = fmaf(rf[c] * uf[c], kf[c], p);
             }
             uint32_t h0, l0, h1, l1;
@@ -428,14 +445,16 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             split2(rhv[0], rhv[1], h0, l0); split2(rhv[2], rhv[3], h1, l1);
             *reinterpret_cast<uint2 *>(&sm.rh[o]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.rhl[o]) = make_uint2(l0, l1);
-            split2(knv[0], knv[1], h0, l0); split2(knv[2], knv[3], h1, l1);
-            *reinterpret_cast<uint2 *>(&sm.kn[o]) = make_uint2(h0, h1);
-            *reinterpret_cast<uint2 *>(&sm.knl[o]) = make_uint2(l0, l1);
             split2(khv[0], khv[1], h0, l0); split2(khv[2], khv[3], h1, l1);
             *reinterpret_cast<uint2 *>(&sm.kh[ot]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.khl[ot]) = make_uint2(l0, l1);
             *reinterpret_cast<uint2 *>(&sm.v[ot]) = pv;
-            if (last_tok) *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+            if ((w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
+                if (g == 3) {
+                    *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+                    *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(__expf(-tot[0]), __expf(-tot[1]), __expf(-tot[2]), __expf(-tot[3]));
+                }
+            }
             p = row_prefix_sum(p);           // lane 15 of the row ends with the sum over the 64 channels
             if (n == 15) sm.rho[tok] = p;
         }
@@ -476,17 +495,19 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             }
         } else if (builder) {
             // ---------------- the masked intra-block matrix of block wv, once for everybody:
-            // A^T[s][t] = sum_i kn[s][i] rh[t][i]; lane gets s = 4g+e, t = n
+            // A^T[s][t] = sum_i (k e^{b-incl})[s][i] (r e^{excl-b})[t][i]; lane gets s = 4g+e, t = n
             const int row = 16 * wv + n;
             f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
 #pragma unroll
             for (int kk = 0; kk < 4; kk += 2) {
                 const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
-                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb);
+                s4 r0, r1, r0l, r1l;
+                scale_split(frag(sm.rh, row, ca), frag(sm.rhl, row, ca), *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), n == 0, r0, r0l);
+                scale_split(frag(sm.rh, row, cb), frag(sm.rhl, row, cb), *reinterpret_cast<const float4 *>(&sm.ent[wv][cb]), n == 0, r1, r1l);
                 a0 = mma2(k0, k1, r0, r1, a0);
-                a1 = mma2(frag(sm.knl, row, ca), frag(sm.knl, row, cb), r0, r1, a1);
-                a2 = mma2(k0, k1, frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), a2);
+                a1 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), r0, r1, a1);
+                a2 = mma2(k0, k1, r0l, r1l, a2);
             }
             f4 at = a0 + (a1 + a2);
             const float rho_t = sm.rho[row];
@@ -515,6 +536,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
 #pragma unroll
             for (int e = 0; e < 4; e++) sm.rh[(16 * q + 4 * g + e) * LD + 16 * wv + n] = bf16_bits(yt[e]);
         }
+        if (sb + 1 < sb1) scan_ahead();      // the next step's w has arrived by now
         PT_MARK(4)
         lds_barrier();
         have_y = y != nullptr;
@@ -693,14 +715,14 @@ struct Bwd16Tiles {
     uint16_t v[SB * LD];     // v               [token][value]
     uint16_t rh[SB * LD];    // r e^{excl}      [token][key]   head / remainder
     uint16_t rhl[SB * LD];
-    uint16_t kn[SB * LD];    // k e^{-incl}     [token][key]
-    uint16_t knl[SB * LD];
     uint16_t kh[SB * LD];    // k e^{b-incl}    [token][key]
     uint16_t khl[SB * LD];
     float incl[SB * HEAD];   // inclusive running log decay inside the block [token][key]
     float lw[SB * HEAD];     // log w                                         [token][key]
+    uint32_t rk[SB * HEAD];  // r and k as they came (bf16 pair: r low, k high)                 [token][key]
     float tot[4][HEAD];      // b per block and key
     float dec[4][HEAD];      // e^{b}
+    float ent[4][HEAD];      // e^{-b}
     float rho[SB];           // r . (u o k) per token
     float wtot[16][HEAD];    // per wavefront (four tokens) and channel: sum of log w, for the block-wide running sum
     float q1[SB * HEAD];     // gy S^T          [token][key]
@@ -778,7 +800,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
 
     // preparing role: token tok of the step (block q), channels c4..c4+3 (one 128-byte row per 16 lanes)
     const int c4 = 4 * n, tok = 4 * w16 + g;
-    const bool last_tok = (w16 & 3) == 3 && g == 3;        // the block's last token
+
     bool have_out = false;
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
@@ -843,13 +865,14 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 for (int c = 0; c < 4; c++) l[c] = log_decay(l[c], floor_decay);
             }
             if (have_out) write_out(sb + 1, tok, c4);
-            block_scan(l, inc, tot, sm.wtot, w16, g, n);
-            float rhv[4], knv[4], khv[4], p = 0.f;
+            scan_local(l, inc, sm.wtot, w16, g, n);      // (the one-step-ahead form of forward16 costs registers this kernel lacks)
+            lds_barrier();
+            scan_join(inc, tot, sm.wtot, w16, n);
+            float rhv[4], khv[4], p = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 rhv[c] = rf[c] * __expf(inc[c] - l[c]);
                 khv[c] = kf[c] * __expf(tot[c] - inc[c]);
-                knv[c] = last_tok ? 0.f : kf[c] * __expf(-inc[c]);     // the block's last token has no later token
                 p = fmaf(rf[c] * uf[c], kf[c], p);
             }
             uint32_t h0, l0, h1, l1;
@@ -859,17 +882,20 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             split2(rhv[0], rhv[1], h0, l0); split2(rhv[2], rhv[3], h1, l1);
             *reinterpret_cast<uint2 *>(&sm.rh[o]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.rhl[o]) = make_uint2(l0, l1);
-            split2(knv[0], knv[1], h0, l0); split2(knv[2], knv[3], h1, l1);
-            *reinterpret_cast<uint2 *>(&sm.kn[o]) = make_uint2(h0, h1);
-            *reinterpret_cast<uint2 *>(&sm.knl[o]) = make_uint2(l0, l1);
             split2(khv[0], khv[1], h0, l0); split2(khv[2], khv[3], h1, l1);
             *reinterpret_cast<uint2 *>(&sm.kh[o]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.khl[o]) = make_uint2(l0, l1);
+            *reinterpret_cast<uint4 *>(&sm.rk[tok * HEAD + c4]) =
+                make_uint4((pr.x & 0xffffu) | (pk.x << 16), (pr.x >> 16) | (pk.x & 0xffff0000u),
+                           (pr.y & 0xffffu) | (pk.y << 16), (pr.y >> 16) | (pk.y & 0xffff0000u));
             *reinterpret_cast<float4 *>(&sm.incl[tok * HEAD + c4]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
             *reinterpret_cast<float4 *>(&sm.lw[tok * HEAD + c4]) = make_float4(l[0], l[1], l[2], l[3]);
-            if (last_tok) {
-                *reinterpret_cast<float4 *>(&sm.tot[q][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
-                *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+            if ((w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
+                if (g == 3) {
+                    *reinterpret_cast<float4 *>(&sm.tot[q][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
+                    *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+                    *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(__expf(-tot[0]), __expf(-tot[1]), __expf(-tot[2]), __expf(-tot[3]));
+                }
             }
             p = row_prefix_sum(p);           // lane 15 of the row ends with the sum over the 64 channels
             if (n == 15) sm.rho[tok] = p;
@@ -997,16 +1023,18 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 sm.pfr[wv][1][lane] = make_uint4(h0, h1, l0, l1);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // A~[t = 4g+e][s = n] = rh_t . kn_s
+            // A~[t = 4g+e][s = n] = (r e^{excl-b})_t . (k e^{b-incl})_s
             f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
 #pragma unroll
             for (int kk = 0; kk < 4; kk += 2) {
                 const int ca = 16 * kk + 4 * g, cb = ca + 16;
-                const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
-                const s4 k0 = frag(sm.kn, row, ca), k1 = frag(sm.kn, row, cb);
+                s4 r0, r1, r0l, r1l;
+                scale_split(frag(sm.rh, row, ca), frag(sm.rhl, row, ca), *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), n == 0, r0, r0l);
+                scale_split(frag(sm.rh, row, cb), frag(sm.rhl, row, cb), *reinterpret_cast<const float4 *>(&sm.ent[wv][cb]), n == 0, r1, r1l);
+                const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb);
                 a0 = mma2(r0, r1, k0, k1, a0);
-                a1 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), k0, k1, a1);
-                a2 = mma2(r0, r1, frag(sm.knl, row, ca), frag(sm.knl, row, cb), a2);
+                a1 = mma2(r0l, r1l, k0, k1, a1);
+                a2 = mma2(r0, r1, frag(sm.khl, row, ca), frag(sm.khl, row, cb), a2);
             }
             f4 at = a0 + (a1 + a2);
             const float rho_s = sm.rho[row];
@@ -1050,7 +1078,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             q2b = mma(pT_h, khTfl, q2b);
             q3b = mma(pm_h, rhTfl, q3b);
             q2 += q2b; q3 += q3b;
-            const float tot_i = sm.tot[q][own], ent_i = __expf(-tot_i);
+            const float tot_i = sm.tot[q][own], ent_i = sm.ent[q][own];
             float c[4], z[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -1058,9 +1086,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
                 const float E1 = __expf(exc), E2 = __expf(tot_i - inc);
                 const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
-                // r, k back from their scaled head + remainder (16 mantissa bits)
-                const float rr = (bf2f(sm.rh[tk * LD + own]) + bf2f(sm.rhl[tk * LD + own])) * __expf(-exc);
-                const float kr = (bf2f(sm.kh[tk * LD + own]) + bf2f(sm.khl[tk * LD + own])) * __expf(inc - tot_i);
+                const uint32_t rkv = sm.rk[tk * HEAD + own];
+                const float rr = bf_lo(rkv), kr = bf_hi(rkv);
                 const float grv = E1 * (q1 + ent_i * q2[e]) + u_i * kr * pd;
                 const float gkn = E2 * (ent_i * q3[e] + q4);
                 const float gkv = gkn + u_i * rr * pd;
@@ -1203,13 +1230,13 @@ static SegPlan plan_segments(int BH, int Tlen) {
     }
     const int sps = (nsb + want - 1) / want;
     const int nseg = (nsb + sps - 1) / sps;
-    // the summary pass: cut each segment into pieces until the pass has two workgroups per CU
-    // (every piece costs one 16 KB summary, so no finer than needed and never below 2 steps)
+    // the summary pass: cut each segment into pieces until the pass has about 1.5 workgroups per CU
+    // (every piece costs one 16 KB summary and a step of the fold, so no finer than needed and never below 2 steps)
     int pps = sps;
     if (nseg == 1) return SegPlan{1, sps, 1, sps};
     if (forced_piece_steps() > 0) pps = std::min(sps, forced_piece_steps());
     else
-        while (pps >= 4 && (long)BH * (nseg - 1) * ((sps + pps - 1) / pps) < 512) pps = (pps + 1) / 2;
+        while (pps >= 4 && (long)BH * (nseg - 1) * ((sps + pps - 1) / pps) < 384) pps = (pps + 1) / 2;
     int m = (sps + pps - 1) / pps;
     if (nseg * m > MAX_SEG) { m = std::max(1, MAX_SEG / nseg); pps = (sps + m - 1) / m; m = (sps + pps - 1) / pps; }
     return SegPlan{nseg, sps, m, pps};
