@@ -150,121 +150,6 @@ struct Gather {
 // handed back (backward).  [key][value] fp32 plus one decay per key.
 constexpr int PART = HEAD * HEAD + HEAD;
 
-// -------------------------------------------------------------- summary passes --
-// Time-parallel split.  One piece (`pps` steps) of the segments 0..nseg-2, from a zero
-// state: what the piece does to a state handed in, S_out = decay o S_in + delta.
-// fold_summaries then chains the pieces into the state at the start of every segment.
-// Four wavefronts; wavefront w owns value columns 16w..16w+15 of the state; a lane
-// prepares eight tokens of a channel pair (running log decay in registers, one
-// shuffle joins the two halves of a block).
-struct StatePassTiles {
-    uint16_t khT[SB * LD];   // k e^{b-incl}     [key][token]   bf16 head of the value
-    uint16_t khTl[SB * LD];  //                                 bf16 remainder
-    uint16_t vT[SB * LD];    // v                [value][token]
-    float dec[4][HEAD];      // e^{b} per block and key
-};
-
-template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_F) void state_pass(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
-        const bf16 *__restrict__ k, const bf16 *__restrict__ v, const float *__restrict__ wraw,
-        float *__restrict__ part, int floor_decay)
-{
-    __shared__ __align__(16) StatePassTiles sm;
-    const int units = (nseg - 1) * m;       // workgroups per (batch, head)
-    const int bh = blockIdx.x / units, unit = blockIdx.x % units, b = bh / H, h = bh % H, seg = unit / m;
-    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
-    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
-    const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = seg * sps + (unit % m) * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
-
-    // state tiles: S[kk][e] = S[key 16kk+4g+e][value 16wv+n]; Dacc = product of the decays
-    f4 S[4], Dacc[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++) {
-        S[kk] = f4{0.f, 0.f, 0.f, 0.f};
-        Dacc[kk] = f4{1.f, 1.f, 1.f, 1.f};
-    }
-    // preparing role: block wv of the step, tokens 8*half..8*half+7 of it, channels c0, c0+1
-    const int half = lane >> 5, c0 = 2 * (lane & 31);
-    float2 l_const = make_float2(0.f, 0.f);
-    if (!PER_TOKEN_W) {
-        l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
-        l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
-    }
-    uint32_t pk[8], pv[8];
-    float2 pw[8];
-    auto fetch = [&](int sb) {
-#pragma unroll
-        for (int x = 0; x < 8; x++) {
-            const int t = sb * SB + 16 * wv + 8 * half + x;
-            if (t < Tlen) {
-                const size_t o = base + (size_t)t * C + c0;
-                pk[x] = *reinterpret_cast<const uint32_t *>(k + o);
-                pv[x] = *reinterpret_cast<const uint32_t *>(v + o);
-                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
-            } else {
-                pk[x] = pv[x] = 0;
-                pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);   // log w = 0
-            }
-        }
-    };
-    if (sb0 < sb1) fetch(sb0);
-    for (int sb = sb0; sb < sb1; sb++) {
-        {
-            float ia[8], ib[8];
-            float ra = 0.f, rb = 0.f;
-#pragma unroll
-            for (int x = 0; x < 8; x++) {
-                ra += PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
-                rb += PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
-                ia[x] = ra; ib[x] = rb;
-            }
-            // the other half of the block sits in lane ^ 32
-            const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
-            const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
-            const float tota = ra + oa, totb = rb + ob;
-            Gather<8> gk_h, gk_l, gv_;
-#pragma unroll
-            for (int x = 0; x < 8; x++) {
-                uint32_t hi, lo;
-                split2(bf_lo(pk[x]) * __expf(tota - (ia[x] + offa)), bf_hi(pk[x]) * __expf(totb - (ib[x] + offb)), hi, lo);
-                gk_h.add(x, hi);
-                gk_l.add(x, lo);
-                gv_.add(x, pv[x]);
-            }
-            const int ot = c0 * LD + 16 * wv + 8 * half;
-            gk_h.put(sm.khT, ot);
-            gk_l.put(sm.khTl, ot);
-            gv_.put(sm.vT, ot);
-            if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(tota), __expf(totb));
-        }
-        lds_barrier();
-        if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const s4 v_op = frag(sm.vT, 16 * wv + n, 16 * q + 4 * g);   // v[s = 4g..][j = 16wv+n]
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
-                S[kk][0] *= d4.x; S[kk][1] *= d4.y; S[kk][2] *= d4.z; S[kk][3] *= d4.w;
-                Dacc[kk][0] *= d4.x; Dacc[kk][1] *= d4.y; Dacc[kk][2] *= d4.z; Dacc[kk][3] *= d4.w;
-                S[kk] = mma2(frag(sm.khT, 16 * kk + n, 16 * q + 4 * g), frag(sm.khTl, 16 * kk + n, 16 * q + 4 * g),
-                             v_op, v_op, S[kk]);
-            }
-        }
-        lds_barrier();
-    }
-    float *pp = part + ((size_t)bh * nseg * m + unit) * PART;
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int row = 16 * kk + 4 * g + e;
-            pp[row * HEAD + 16 * wv + n] = S[kk][e];
-            if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
-        }
-}
-
 // ------------------------------------------------------- forward, 16 wavefronts --
 // The main forward pass with the work of a 64-token step spread over 16 wavefronts
 // (four per SIMD).  A step runs in three phases separated by workgroup barriers:
@@ -347,6 +232,142 @@ __device__ __forceinline__ void scan_join(float (&inc)[4], float (&tot)[4], cons
         tot[0] += t4.x; tot[1] += t4.y; tot[2] += t4.z; tot[3] += t4.w;
         if (x < pos) { inc[0] += t4.x; inc[1] += t4.y; inc[2] += t4.z; inc[3] += t4.w; }
     }
+}
+
+// -------------------------------------------------------------- summary passes --
+// Time-parallel split.  One piece (`pps` steps) of a segment, from a zero state
+// (gradient): what the piece does to a state handed in, X_out = decay o X_in + delta.
+//   BACKWARD = false: state summary over pieces of the segments 0..nseg-2 (reads k, v, w):
+//                     X <- e^{b} o X + (k e^{b-incl})^T v      per 16-token block, first to last;
+//   BACKWARD = true:  state-gradient summary over pieces of the segments 1..nseg-1 (reads r, gy, w):
+//                     X <- e^{b} o X + (r e^{excl})^T gy       per 16-token block, last to first.
+// fold_summaries then chains the pieces.  Four wavefronts; wavefront w prepares block w of
+// a step (lane = four consecutive tokens x four channels, 16 lanes = one 128-byte row, the
+// running log decay inside the lane and two shuffles across) and owns value columns
+// 16w..16w+15 of X.  Tiles are [token][channel]; the MFMA operands come out of the
+// transposing LDS read.
+struct PassTiles {
+    uint16_t a[SB * LD];      // forward: k e^{b-incl};  backward: r e^{excl}     [token][key]   bf16 head of the value
+    uint16_t al[SB * LD];     //                                                                 bf16 remainder
+    uint16_t b[SB * LD];      // forward: v;             backward: gy             [token][value]
+    float dec[4][HEAD];       // e^{b} per block and key
+    float tot[4][HEAD];       // b
+};
+
+template <bool PER_TOKEN_W, bool BACKWARD>
+__global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
+        const bf16 *__restrict__ a_in, const bf16 *__restrict__ b_in, const float *__restrict__ wraw,
+        float *__restrict__ part, int floor_decay)
+{
+    __shared__ __align__(16) PassTiles sm;
+    const int units = (nseg - 1) * m;       // workgroups per (batch, head)
+    const int bh = blockIdx.x / units, piece = (BACKWARD ? m : 0) + blockIdx.x % units, seg = piece / m, b = bh / H, h = bh % H;
+    const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    const int nsb = (Tlen + SB - 1) / SB;
+    const int sb0 = seg * sps + (piece % m) * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
+    const int nsteps = sb1 - sb0;
+
+    // X[kk][e] = X[key 16kk+4g+e][value 16wv+n]
+    f4 X[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) X[kk] = f4{0.f, 0.f, 0.f, 0.f};
+    float dsum = 0.f;                       // wavefront 0, lane = key: log of the piece's decay
+    // preparing role: tokens tok0..tok0+3 of the step (block wv), channels c4..c4+3
+    const int c4 = 4 * n, tok0 = 16 * wv + 4 * g;
+    float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!PER_TOKEN_W) {
+        const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+        l_const = make_float4(log_decay(w4.x, floor_decay), log_decay(w4.y, floor_decay), log_decay(w4.z, floor_decay),
+                              log_decay(w4.w, floor_decay));
+    }
+    uint2 pa[4], pb[4];
+    float4 pw[4];
+    auto fetch = [&](int sb) {
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+            const int t = sb * SB + tok0 + x;
+            if (t < Tlen) {
+                const size_t o = base + (size_t)t * C + c4;
+                pa[x] = *reinterpret_cast<const uint2 *>(a_in + o);
+                pb[x] = *reinterpret_cast<const uint2 *>(b_in + o);
+                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+            } else {
+                pa[x] = pb[x] = make_uint2(0u, 0u);
+                pw[x] = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    };
+    const int tro = tr_lane_offset(lane, LD);
+    if (nsteps > 0) fetch(BACKWARD ? sb1 - 1 : sb0);
+    for (int it = 0; it < nsteps; it++) {
+        const int sb = BACKWARD ? sb1 - 1 - it : sb0 + it;
+        {
+            float l[4][4], inc[4][4], run[4] = {0.f, 0.f, 0.f, 0.f}, tot[4];
+#pragma unroll
+            for (int x = 0; x < 4; x++) {
+                const float lw4[4] = {pw[x].x, pw[x].y, pw[x].z, pw[x].w};
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    l[x][c] = PER_TOKEN_W ? log_decay(lw4[c], floor_decay) : lw4[c];
+                    run[c] += l[x][c];
+                    inc[x][c] = run[c];
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) {          // the lanes g-1, g-2, g-3 hold the earlier tokens of the block
+                float x = run[c];
+                const float u1 = __shfl_up(x, 16);
+                x += g >= 1 ? u1 : 0.f;
+                const float u2 = __shfl_up(x, 32);
+                x += g >= 2 ? u2 : 0.f;
+                tot[c] = __shfl(x, lane | 48);
+                run[c] = x - run[c];               // what comes before this lane's tokens
+            }
+#pragma unroll
+            for (int x = 0; x < 4; x++) {
+                const float af[4] = {bf_lo(pa[x].x), bf_hi(pa[x].x), bf_lo(pa[x].y), bf_hi(pa[x].y)};
+                float sc[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const float ic = inc[x][c] + run[c];
+                    sc[c] = af[c] * __expf(BACKWARD ? ic - l[x][c] : tot[c] - ic);       // r e^{excl}  /  k e^{b-incl}
+                }
+                uint32_t h0, l0, h1, l1;
+                const int o = (tok0 + x) * LD + c4;
+                split2(sc[0], sc[1], h0, l0); split2(sc[2], sc[3], h1, l1);
+                *reinterpret_cast<uint2 *>(&sm.a[o]) = make_uint2(h0, h1);
+                *reinterpret_cast<uint2 *>(&sm.al[o]) = make_uint2(l0, l1);
+                *reinterpret_cast<uint2 *>(&sm.b[o]) = pb[x];
+            }
+            if (g == 3) {
+                *reinterpret_cast<float4 *>(&sm.tot[wv][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
+                *reinterpret_cast<float4 *>(&sm.dec[wv][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+            }
+        }
+        lds_barrier();
+        if (it + 1 < nsteps) fetch(BACKWARD ? sb - 1 : sb + 1);          // next step's loads fly during the MFMA phase
+        if (wv == 0) dsum += (sm.tot[0][lane] + sm.tot[1][lane]) + (sm.tot[2][lane] + sm.tot[3][lane]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int blk = BACKWARD ? 3 - i : i;
+            const s4 b_op = frag_tr(sm.b, tro + (16 * blk) * LD + 16 * wv);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][16 * kk + 4 * g]);
+                X[kk][0] *= d4.x; X[kk][1] *= d4.y; X[kk][2] *= d4.z; X[kk][3] *= d4.w;
+                X[kk] = mma2(frag_tr(sm.a, tro + (16 * blk) * LD + 16 * kk), frag_tr(sm.al, tro + (16 * blk) * LD + 16 * kk),
+                             b_op, b_op, X[kk]);
+            }
+        }
+        lds_barrier();
+    }
+    float *pp = part + ((size_t)bh * nseg * m + piece) * PART;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) pp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = X[kk][e];
+    if (wv == 0) pp[HEAD * HEAD + lane] = __expf(dsum);
 }
 
 template <bool PER_TOKEN_W>
@@ -560,117 +581,6 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
                 for (int e = 0; e < 4; e++) op[(32 * hk + 16 * j + 4 * g + e) * HEAD + 16 * wv + n] = S[j][e];
         }
     }
-}
-
-// ------------------------------------------------------------------ backward --
-// State-gradient summary of one piece (`pps` steps) of the segments 1..nseg-1 for the
-// backward split: from a zero gradient, walks the piece's tokens last to first with
-//   G <- e^{b} o G + (r e^{excl})^T gy      per 16-token block
-// and leaves  delta = G, decay = product of e^{b}  in gpart; fold_backward turns the
-// summaries into the gradient at the end of every segment.  One wavefront per 16 value
-// columns, as the forward's state.
-struct GPassTiles {
-    uint16_t rhT[SB * LD];   // r e^{excl}   [key][token]  head / remainder
-    uint16_t rhTl[SB * LD];
-    uint16_t gyT[SB * LD];   // gy           [value][token]
-    float dec[4][HEAD];
-};
-
-template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_F) void gradient_pass(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
-        const bf16 *__restrict__ r, const float *__restrict__ wraw, const bf16 *__restrict__ gy,
-        float *__restrict__ gpart, int floor_decay)
-{
-    __shared__ __align__(16) GPassTiles sm;
-    const int units = (nseg - 1) * m;
-    const int bh = blockIdx.x / units, piece = m + blockIdx.x % units, seg = piece / m, b = bh / H, h = bh % H;
-    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
-    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
-    const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = seg * sps + (piece % m) * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
-    const int half = lane >> 5, c0 = 2 * (lane & 31);
-    float2 l_const = make_float2(0.f, 0.f);
-    if (!PER_TOKEN_W) {
-        l_const.x = log_decay(wraw[h * HEAD + c0], floor_decay);
-        l_const.y = log_decay(wraw[h * HEAD + c0 + 1], floor_decay);
-    }
-    f4 G[4], Dacc[4];           // G[kk][e] = G[key 16kk+4g+e][value 16wv+n]
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++) {
-        G[kk] = f4{0.f, 0.f, 0.f, 0.f};
-        Dacc[kk] = f4{1.f, 1.f, 1.f, 1.f};
-    }
-    uint32_t pr[8], pg[8];
-    float2 pw[8];
-    auto fetch = [&](int sb) {
-#pragma unroll
-        for (int x = 0; x < 8; x++) {
-            const int t = sb * SB + 16 * wv + 8 * half + x;
-            if (t < Tlen) {
-                const size_t o = base + (size_t)t * C + c0;
-                pr[x] = *reinterpret_cast<const uint32_t *>(r + o);
-                pg[x] = *reinterpret_cast<const uint32_t *>(gy + o);
-                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float2 *>(wraw + o) : l_const;
-            } else {
-                pr[x] = pg[x] = 0;
-                pw[x] = PER_TOKEN_W ? make_float2(-INFINITY, -INFINITY) : make_float2(0.f, 0.f);
-            }
-        }
-    };
-    fetch(sb1 - 1);
-    for (int sb = sb1 - 1; sb >= sb0; sb--) {
-        {
-            float ea[8], eb[8];                 // exclusive running log decay inside this lane's 8 tokens
-            float ra = 0.f, rb = 0.f;
-#pragma unroll
-            for (int x = 0; x < 8; x++) {
-                ea[x] = ra; eb[x] = rb;
-                ra += PER_TOKEN_W ? log_decay(pw[x].x, floor_decay) : pw[x].x;
-                rb += PER_TOKEN_W ? log_decay(pw[x].y, floor_decay) : pw[x].y;
-            }
-            const float oa = __shfl_xor(ra, 32), ob = __shfl_xor(rb, 32);
-            const float offa = half ? oa : 0.f, offb = half ? ob : 0.f;
-            Gather<8> gr_h, gr_l, gg_;
-#pragma unroll
-            for (int x = 0; x < 8; x++) {
-                uint32_t hi, lo;
-                split2(bf_lo(pr[x]) * __expf(ea[x] + offa), bf_hi(pr[x]) * __expf(eb[x] + offb), hi, lo);
-                gr_h.add(x, hi);
-                gr_l.add(x, lo);
-                gg_.add(x, pg[x]);
-            }
-            const int ot = c0 * LD + 16 * wv + 8 * half;
-            gr_h.put(sm.rhT, ot);
-            gr_l.put(sm.rhTl, ot);
-            gg_.put(sm.gyT, ot);
-            if (!half) *reinterpret_cast<float2 *>(&sm.dec[wv][c0]) = make_float2(__expf(ra + oa), __expf(rb + ob));
-        }
-        lds_barrier();
-        if (sb > sb0) fetch(sb - 1);
-#pragma unroll
-        for (int q = 3; q >= 0; q--) {
-            if (sb * SB + 16 * q >= Tlen) continue;
-            const s4 gyTf = frag(sm.gyT, 16 * wv + n, 16 * q + 4 * g);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[q][16 * kk + 4 * g]);
-                G[kk][0] *= d4.x; G[kk][1] *= d4.y; G[kk][2] *= d4.z; G[kk][3] *= d4.w;
-                Dacc[kk][0] *= d4.x; Dacc[kk][1] *= d4.y; Dacc[kk][2] *= d4.z; Dacc[kk][3] *= d4.w;
-                G[kk] = mma2(frag(sm.rhT, 16 * kk + n, 16 * q + 4 * g), frag(sm.rhTl, 16 * kk + n, 16 * q + 4 * g),
-                             gyTf, gyTf, G[kk]);
-            }
-        }
-        lds_barrier();
-    }
-    float *pp = gpart + ((size_t)bh * nseg * m + piece) * PART;
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int row = 16 * kk + 4 * g + e;
-            pp[row * HEAD + 16 * wv + n] = G[kk][e];
-            if (wv == 0 && n == 0) pp[HEAD * HEAD + row] = Dacc[kk][e];
-        }
 }
 
 // ------------------------------------------------------ backward, 16 wavefronts --
@@ -1276,11 +1186,11 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
         const int pieces = (pl.nseg - 1) * pl.m;
         dim3 grid(B * H * pieces);
         if (per_token)
-            hipLaunchKernelGGL((state_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w, part,
-                               floor_decay);
+            hipLaunchKernelGGL((summary_pass<true, false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w,
+                               part, floor_decay);
         else
-            hipLaunchKernelGGL((state_pass<false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w, part,
-                               floor_decay);
+            hipLaunchKernelGGL((summary_pass<false, false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w,
+                               part, floor_decay);
         hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, 0, pieces - 1, 1, pl.m,
                            pl.nseg * pl.m, s_in, part);
         hipError_t e = hipGetLastError();
@@ -1324,11 +1234,11 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
         const int pieces = (pl.nseg - 1) * pl.m;
         dim3 grid(B * H * pieces), block(NT_F);
         if (per_token)
-            hipLaunchKernelGGL((gradient_pass<true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, w,
-                               gg, gpart, floor_decay);
+            hipLaunchKernelGGL((summary_pass<true, true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, gg, w,
+                               gpart, floor_decay);
         else
-            hipLaunchKernelGGL((gradient_pass<false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, w,
-                               gg, gpart, floor_decay);
+            hipLaunchKernelGGL((summary_pass<false, true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, gg, w,
+                               gpart, floor_decay);
         hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, pl.nseg * pl.m - 1, pl.m,
                            -1, pl.m, pl.nseg * pl.m, gs_out, gpart);
         hipError_t e = hipGetLastError();
