@@ -818,7 +818,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
         f4 KG[4];                    // wavefronts 8-11: kh G per block, KG[q][e] at [token 4g+e][value own]
       {
         WKV_LOCAL_LANE
-        if (sb > sb0) fetch(sb - 1, tok, c4);
         if (role == 0) {
             // ---------------- state chain, first block to last; Q1[t][key own] = sum_j gy[t][j] S[key own][j]
 #pragma unroll
@@ -957,6 +956,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             split2(at[0], at[1], h0, l0); split2(at[2], at[3], h1, l1);
             sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
         }
+        if (sb > sb0) fetch(sb - 1, tok, c4);      // after the chains: they are short of registers
       }
         PT_MARK(2)
         lds_barrier();
