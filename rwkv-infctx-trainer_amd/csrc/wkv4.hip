@@ -1,9 +1,11 @@
 // RWKV-v4 WKV with (aa, bb, pp) state: one lane per (batch, channel) chain.
 //
 // The chain is serial in time, so the kernels keep many independent loads in
-// flight per lane instead: a block of 16 tokens of k, v (and gy) is fetched
-// into registers while the previous block is consumed; consecutive lanes are
-// consecutive channels, so every load and store is a full coalesced row.
+// flight per lane instead: blocks of 16 tokens of k, v (and gy) are fetched
+// into registers two (backward: one) blocks ahead of the one being consumed;
+// consecutive lanes are consecutive channels, so every load and store is a full
+// coalesced row.  The speed is set by one wavefront's walk over T (about 450
+// cycles per token forward): partly filled wavefronts on more SIMDs do not help.
 //
 // State convention (RWKV-v4neo/cuda/wkv_cuda_bf16.cu:30-52): (p, q, o) with
 // p, q the decayed sums divided by e^{o}.  Backward carries the state gradient
@@ -57,7 +59,10 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
     Chain s{0.f, 0.f, NEG_HUGE, 0.f, 0.f};
     if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
 
-    float ck[CK], cv[CK], nk[CK], nv[CK];
+    // three 16-token blocks of k, v per lane: one being consumed, two in flight (a chain is serial and a CU holds
+    // few chains, so the bytes in flight per lane are what sets the bandwidth); indexed statically by unrolling
+    constexpr int RING = 3;
+    float bk[RING][CK], bv[RING][CK];
     auto fetch = [&](int t0, float (&kk)[CK], float (&vv)[CK]) {
 #pragma unroll
         for (int i = 0; i < CK; i++) {
@@ -66,23 +71,28 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
             vv[i] = in ? to_float(v[base + (size_t)(t0 + i) * C]) : 0.f;
         }
     };
-    fetch(0, ck, cv);
-    for (int t0 = 0, blk = 0; t0 < Tlen; t0 += CK, blk++) {
-        if (t0 + CK < Tlen) fetch(t0 + CK, nk, nv);
-        if (ckpt) {
-            float *cp = ckpt + (size_t)blk * 5 * BC + idx;
-            cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
-        }
 #pragma unroll
-        for (int i = 0; i < CK; i++) {
-            if (t0 + i < Tlen) {
-                float iden, cexp, hw;
-                const float yy = v4_step(s, w, u, ck[i], cv[i], iden, cexp, hw);
-                if (y) y[base + (size_t)(t0 + i) * C] = from_float<T>(yy);
+    for (int d = 0; d < RING; d++)
+        if (d * CK < Tlen) fetch(d * CK, bk[d], bv[d]);
+    for (int tb = 0, blk = 0; tb < Tlen; tb += RING * CK) {
+#pragma unroll
+        for (int d = 0; d < RING; d++, blk++) {
+            const int t0 = tb + d * CK;
+            if (t0 >= Tlen) break;
+            if (ckpt) {
+                float *cp = ckpt + (size_t)blk * 5 * BC + idx;
+                cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
             }
-        }
 #pragma unroll
-        for (int i = 0; i < CK; i++) { ck[i] = nk[i]; cv[i] = nv[i]; }
+            for (int i = 0; i < CK; i++) {
+                if (t0 + i < Tlen) {
+                    float iden, cexp, hw;
+                    const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, cexp, hw);
+                    if (y) y[base + (size_t)(t0 + i) * C] = from_float<T>(yy);
+                }
+            }
+            if (t0 + RING * CK < Tlen) fetch(t0 + RING * CK, bk[d], bv[d]);
+        }
     }
     if (s_out) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
 }
@@ -102,9 +112,12 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
 
     float gp = 0.f, gq = 0.f, go = NEG_HUGE, acc_w = 0.f, acc_u = 0.f;
     const int nblk = (Tlen + CK - 1) / CK;
-    for (int blk = nblk - 1; blk >= 0; blk--) {
+    // two blocks of k, v, gy and their checkpoints per lane: one being consumed, one in flight
+    constexpr int RING = 2;
+    float bk[RING][CK], bv[RING][CK], bg[RING][CK];
+    Chain bs[RING];
+    auto fetch = [&](int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain &cs) {
         const int t0 = blk * CK;
-        float kk[CK], vv[CK], gg[CK], ys[CK], iden[CK], cexp[CK];
 #pragma unroll
         for (int i = 0; i < CK; i++) {
             const bool in = t0 + i < Tlen;
@@ -114,7 +127,20 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
             gg[i] = in ? to_float(gy[o]) : 0.f;
         }
         const float *cp = ckpt + (size_t)blk * 5 * BC + idx;
-        Chain s{cp[0], cp[BC], cp[2 * (size_t)BC], cp[3 * (size_t)BC], cp[4 * (size_t)BC]};
+        cs = Chain{cp[0], cp[BC], cp[2 * (size_t)BC], cp[3 * (size_t)BC], cp[4 * (size_t)BC]};
+    };
+#pragma unroll
+    for (int d = 0; d < RING; d++)
+        if (nblk - 1 - d >= 0) fetch(nblk - 1 - d, bk[d], bv[d], bg[d], bs[d]);
+    for (int bb = nblk - 1; bb >= 0; bb -= RING) {
+#pragma unroll
+      for (int d = 0; d < RING; d++) {
+        const int blk = bb - d;
+        if (blk < 0) break;
+        const int t0 = blk * CK;
+        float (&kk)[CK] = bk[d], (&vv)[CK] = bv[d], (&gg)[CK] = bg[d];
+        float ys[CK], iden[CK], cexp[CK];
+        Chain s = bs[d];
         // replay the block forward
 #pragma unroll
         for (int i = 0; i < CK; i++) {
@@ -149,6 +175,8 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
                 go = m;
             }
         }
+        if (blk - RING >= 0) fetch(blk - RING, bk[d], bv[d], bg[d], bs[d]);
+      }
     }
     if (gs_in) { gs_in[idx * 3] = gp; gs_in[idx * 3 + 1] = gq; gs_in[idx * 3 + 2] = go; }
     gw_part[idx] = acc_w * w;
