@@ -17,6 +17,7 @@
 // 5-float checkpoint (p, q, o, dp/dw, dq/dw) every 16 tokens, and the backward
 // sweep replays one 16-token block at a time from its checkpoint.
 #include "common.h"
+#include <type_traits>
 
 namespace wkv {
 
@@ -64,11 +65,17 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
     constexpr int RING = 3;
     float bk[RING][CK], bv[RING][CK];
     auto fetch = [&](int t0, float (&kk)[CK], float (&vv)[CK]) {
+        const T *kp = k + base + (size_t)t0 * C, *vp = v + base + (size_t)t0 * C;
+        if (t0 + CK <= Tlen) {          // whole block inside the sequence: no per-token checks
 #pragma unroll
-        for (int i = 0; i < CK; i++) {
-            const bool in = t0 + i < Tlen;
-            kk[i] = in ? to_float(k[base + (size_t)(t0 + i) * C]) : 0.f;
-            vv[i] = in ? to_float(v[base + (size_t)(t0 + i) * C]) : 0.f;
+            for (int i = 0; i < CK; i++, kp += C, vp += C) { kk[i] = to_float(*kp); vv[i] = to_float(*vp); }
+        } else {
+#pragma unroll
+            for (int i = 0; i < CK; i++, kp += C, vp += C) {
+                const bool in = t0 + i < Tlen;
+                kk[i] = in ? to_float(*kp) : 0.f;
+                vv[i] = in ? to_float(*vp) : 0.f;
+            }
         }
     };
 #pragma unroll
@@ -83,12 +90,23 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
                 float *cp = ckpt + (size_t)blk * 5 * BC + idx;
                 cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
             }
+            T *yp = y ? y + base + (size_t)t0 * C : nullptr;
+            const int cnt = min(CK, Tlen - t0);
+            if (cnt == CK) {
 #pragma unroll
-            for (int i = 0; i < CK; i++) {
-                if (t0 + i < Tlen) {
+                for (int i = 0; i < CK; i++) {
                     float iden, cexp, hw;
                     const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, cexp, hw);
-                    if (y) y[base + (size_t)(t0 + i) * C] = from_float<T>(yy);
+                    if (yp) { *yp = from_float<T>(yy); yp += C; }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < CK; i++) {
+                    if (i < cnt) {
+                        float iden, cexp, hw;
+                        const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, cexp, hw);
+                        if (yp) { *yp = from_float<T>(yy); yp += C; }
+                    }
                 }
             }
             if (t0 + RING * CK < Tlen) fetch(t0 + RING * CK, bk[d], bv[d]);
@@ -118,33 +136,31 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
     Chain bs[RING];
     auto fetch = [&](int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain &cs) {
         const int t0 = blk * CK;
+        const size_t o0 = base + (size_t)t0 * C;
+        const T *kp = k + o0, *vp = v + o0, *gp_ = gy + o0;
+        if (t0 + CK <= Tlen) {          // whole block inside the sequence: no per-token checks
 #pragma unroll
-        for (int i = 0; i < CK; i++) {
-            const bool in = t0 + i < Tlen;
-            const size_t o = base + (size_t)(t0 + i) * C;
-            kk[i] = in ? to_float(k[o]) : 0.f;
-            vv[i] = in ? to_float(v[o]) : 0.f;
-            gg[i] = in ? to_float(gy[o]) : 0.f;
+            for (int i = 0; i < CK; i++, kp += C, vp += C, gp_ += C) { kk[i] = to_float(*kp); vv[i] = to_float(*vp); gg[i] = to_float(*gp_); }
+        } else {
+#pragma unroll
+            for (int i = 0; i < CK; i++, kp += C, vp += C, gp_ += C) {
+                const bool in = t0 + i < Tlen;
+                kk[i] = in ? to_float(*kp) : 0.f;
+                vv[i] = in ? to_float(*vp) : 0.f;
+                gg[i] = in ? to_float(*gp_) : 0.f;
+            }
         }
         const float *cp = ckpt + (size_t)blk * 5 * BC + idx;
         cs = Chain{cp[0], cp[BC], cp[2 * (size_t)BC], cp[3 * (size_t)BC], cp[4 * (size_t)BC]};
     };
-#pragma unroll
-    for (int d = 0; d < RING; d++)
-        if (nblk - 1 - d >= 0) fetch(nblk - 1 - d, bk[d], bv[d], bg[d], bs[d]);
-    for (int bb = nblk - 1; bb >= 0; bb -= RING) {
-#pragma unroll
-      for (int d = 0; d < RING; d++) {
-        const int blk = bb - d;
-        if (blk < 0) break;
-        const int t0 = blk * CK;
-        float (&kk)[CK] = bk[d], (&vv)[CK] = bv[d], (&gg)[CK] = bg[d];
+    // one block: replay it forward from its checkpoint, then walk it backwards (FULL: all CK tokens exist)
+    auto block = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain s) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        const int t0 = blk * CK, cnt = FULL ? CK : Tlen - t0;
         float ys[CK], iden[CK], cexp[CK];
-        Chain s = bs[d];
-        // replay the block forward
 #pragma unroll
         for (int i = 0; i < CK; i++) {
-            if (t0 + i < Tlen) {
+            if (FULL || i < cnt) {
                 const float dp0 = s.dp, dq0 = s.dq;
                 float hw;
                 ys[i] = v4_step(s, w, u, kk[i], vv[i], iden[i], cexp[i], hw);
@@ -157,15 +173,15 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
             if (gp == 0.f && gq == 0.f) go = NEG_HUGE;
             acc_w += (gp * s.dp + gq * s.dq) * __expf(s.o + go);
         }
-        // and walk it backwards
+        const size_t oe = base + (size_t)(t0 + CK - 1) * C;
+        T *gkp = gk + oe, *gvp = gv + oe;
 #pragma unroll
-        for (int i = CK - 1; i >= 0; i--) {
-            if (t0 + i < Tlen) {
-                const size_t o = base + (size_t)(t0 + i) * C;
+        for (int i = CK - 1; i >= 0; i--, gkp -= C, gvp -= C) {
+            if (FULL || i < cnt) {
                 const float direct = gg[i] * iden[i] * __expf(cexp[i]);
                 const float later = __expf(kk[i] + go);
-                gk[o] = from_float<T>(direct * (vv[i] - ys[i]) + later * (gp * vv[i] + gq));
-                gv[o] = from_float<T>(direct + later * gp);
+                *gkp = from_float<T>(direct * (vv[i] - ys[i]) + later * (gp * vv[i] + gq));
+                *gvp = from_float<T>(direct + later * gp);
                 const float hist = cexp[i] - kk[i] - u;
                 const float m = fmaxf(w + go, hist);
                 const float keep = __expf(w + go - m);
@@ -175,8 +191,19 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
                 go = m;
             }
         }
-        if (blk - RING >= 0) fetch(blk - RING, bk[d], bv[d], bg[d], bs[d]);
-      }
+    };
+#pragma unroll
+    for (int d = 0; d < RING; d++)
+        if (nblk - 1 - d >= 0) fetch(nblk - 1 - d, bk[d], bv[d], bg[d], bs[d]);
+    for (int bb = nblk - 1; bb >= 0; bb -= RING) {
+#pragma unroll
+        for (int d = 0; d < RING; d++) {
+            const int blk = bb - d;
+            if (blk < 0) break;
+            if ((blk + 1) * CK <= Tlen) block(std::true_type{}, blk, bk[d], bv[d], bg[d], bs[d]);
+            else block(std::false_type{}, blk, bk[d], bv[d], bg[d], bs[d]);
+            if (blk - RING >= 0) fetch(blk - RING, bk[d], bv[d], bg[d], bs[d]);
+        }
     }
     if (gs_in) { gs_in[idx * 3] = gp; gs_in[idx * 3 + 1] = gq; gs_in[idx * 3 + 2] = go; }
     gw_part[idx] = acc_w * w;
