@@ -643,6 +643,7 @@ struct Bwd16Tiles {
     float tots[4][HEAD];     // per block and key: sum over the block's tokens of r gr - k gk
     float arun[HEAD];        // the running sum at the end of the current step
     float red[2][4][HEAD];   // gu / gw partial sums of the four block groups
+    float4 kg3[4][64];       // kh G of the step's last block, parked here by wavefronts 8-11 (they are short of registers)
 };
 constexpr int NT_B16 = 1024;
 // Re-derives the lane-dependent indices from an opaque copy of the lane id, so that the
@@ -890,6 +891,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                     g2 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g2);
                 }
                 KG[qq] = g0 + (g1 + g2);
+                if (qq == 3) sm.kg3[wv][lane] = make_float4(KG[3][0], KG[3][1], KG[3][2], KG[3][3]);
                 const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
 #pragma unroll
                 for (int kk = 0; kk < 4; kk++) {      // G <- e^{b} o G + rh^T gy
@@ -971,7 +973,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             for (int qq = 0; qq < 4; qq++) {
                 const uint4 am = sm.amat[qq][lane];
                 const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
-                const f4 gvt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), gyTf, gyTf, KG[qq]);
+                f4 kgq = KG[qq < 3 ? qq : 0];
+                if (qq == 3) { const float4 t4 = sm.kg3[wv][lane]; kgq = f4{t4.x, t4.y, t4.z, t4.w}; }
+                const f4 gvt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), gyTf, gyTf, kgq);
 #pragma unroll
                 for (int e = 0; e < 4; e++) sm.v[(16 * qq + 4 * g + e) * LD + own] = bf16_bits(gvt[e]);      // v is not read any more
             }
