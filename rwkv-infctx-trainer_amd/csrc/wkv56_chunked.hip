@@ -823,17 +823,16 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             // ---------------- state chain, first block to last; Q1[t][key own] = sum_j gy[t][j] S[key own][j]
 #pragma unroll
             for (int qq = 0; qq < 4; qq++) {
-                f4 qa = {0.f, 0.f, 0.f, 0.f}, qb = qa;
+                f4 qa = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kk = 0; kk < 4; kk += 2) {
                     s4 s0h, s0l, s1h, s1l;
                     split4(G[kk], s0h, s0l);
                     split4(G[kk + 1], s1h, s1l);
                     const s4 y0 = frag(sm.gy, 16 * qq + n, 16 * kk + 4 * g), y1 = frag(sm.gy, 16 * qq + n, 16 * kk + 16 + 4 * g);
+                    qa = mma2(y0, y1, s0l, s1l, qa);
                     qa = mma2(y0, y1, s0h, s1h, qa);
-                    qb = mma2(y0, y1, s0l, s1l, qb);
                 }
-                qa += qb;
 #pragma unroll
                 for (int e = 0; e < 4; e++) sm.q1[(16 * qq + 4 * g + e) * HEAD + own] = qa[e];
                 if (qq < 3) {
@@ -851,17 +850,16 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             // ---------------- state-gradient chain (value-major), last block to first; Q4[s][key own] = sum_j v[s][j] G[key own][j]
 #pragma unroll
             for (int qq = 3; qq >= 0; qq--) {
-                f4 q4 = {0.f, 0.f, 0.f, 0.f}, q4b = q4;
+                f4 q4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kk = 0; kk < 4; kk += 2) {
                     s4 g0h, g0l, g1h, g1l;
                     split4(G[kk], g0h, g0l);
                     split4(G[kk + 1], g1h, g1l);
                     const s4 v0 = frag(sm.v, 16 * qq + n, 16 * kk + 4 * g), v1 = frag(sm.v, 16 * qq + n, 16 * kk + 16 + 4 * g);
+                    q4 = mma2(v0, v1, g0l, g1l, q4);
                     q4 = mma2(v0, v1, g0h, g1h, q4);
-                    q4b = mma2(v0, v1, g0l, g1l, q4b);
                 }
-                q4 += q4b;
 #pragma unroll
                 for (int e = 0; e < 4; e++) sm.q4[(16 * qq + 4 * g + e) * HEAD + own] = q4[e];
                 const float dq = sm.dec[qq][own];
@@ -878,7 +876,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
 #pragma unroll
             for (int qq = 3; qq >= 0; qq--) {
                 const int row = 16 * qq + n;
-                f4 g0 = {0.f, 0.f, 0.f, 0.f}, g1 = g0, g2 = g0;
+                f4 g0 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kk = 0; kk < 4; kk += 2) {
                     const int ca = 16 * kk + 4 * g, cb = ca + 16;
@@ -886,11 +884,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                     split4(G[kk], g0h, g0l);
                     split4(G[kk + 1], g1h, g1l);
                     const s4 h0 = frag(sm.kh, row, ca), h1 = frag(sm.kh, row, cb);
+                    g0 = mma2(h0, h1, g0l, g1l, g0);
+                    g0 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g0);
                     g0 = mma2(h0, h1, g0h, g1h, g0);
-                    g1 = mma2(h0, h1, g0l, g1l, g1);
-                    g2 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g2);
                 }
-                KG[qq] = g0 + (g1 + g2);
+                KG[qq] = g0;
                 if (qq == 3) sm.kg3[wv][lane] = make_float4(KG[3][0], KG[3][1], KG[3][2], KG[3][3]);
                 const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
 #pragma unroll
@@ -935,7 +933,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             }
             __builtin_amdgcn_sched_barrier(0);
             // A~[t = 4g+e][s = n] = (r e^{excl-b})_t . (k e^{b-incl})_s
-            f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
+            f4 at = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < 4; kk += 2) {
                 const int ca = 16 * kk + 4 * g, cb = ca + 16;
@@ -943,11 +941,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 scale_split(frag(sm.rh, row, ca), frag(sm.rhl, row, ca), *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), n == 0, r0, r0l);
                 scale_split(frag(sm.rh, row, cb), frag(sm.rhl, row, cb), *reinterpret_cast<const float4 *>(&sm.ent[wv][cb]), n == 0, r1, r1l);
                 const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb);
-                a0 = mma2(r0, r1, k0, k1, a0);
-                a1 = mma2(r0l, r1l, k0, k1, a1);
-                a2 = mma2(r0, r1, frag(sm.khl, row, ca), frag(sm.khl, row, cb), a2);
+                at = mma2(r0l, r1l, k0, k1, at);
+                at = mma2(r0, r1, frag(sm.khl, row, ca), frag(sm.khl, row, cb), at);
+                at = mma2(r0, r1, k0, k1, at);
             }
-            f4 at = a0 + (a1 + a2);
             const float rho_s = sm.rho[row];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -986,12 +983,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             const s4 pT_h = as_s4(pa.x, pa.y), pT_l = as_s4(pa.z, pa.w), pm_h = as_s4(pb.x, pb.y), pm_l = as_s4(pb.z, pb.w);
             const s4 khTf = frag_tr(sm.kh, tro + (16 * q) * LD + 16 * wv), khTfl = frag_tr(sm.khl, tro + (16 * q) * LD + 16 * wv);
             const s4 rhTf = frag_tr(sm.rh, tro + (16 * q) * LD + 16 * wv), rhTfl = frag_tr(sm.rhl, tro + (16 * q) * LD + 16 * wv);
-            f4 q2 = {0.f, 0.f, 0.f, 0.f}, q2b = q2, q3 = q2, q3b = q2;
+            f4 q2 = {0.f, 0.f, 0.f, 0.f}, q3 = q2;
+            q2 = mma(pT_h, khTfl, q2);
+            q3 = mma(pm_h, rhTfl, q3);
             q2 = mma2(pT_h, pT_l, khTf, khTf, q2);      // sum_{s<t} P[t][s] kh_s
             q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);      // sum_{t>s} P[t][s] rh_t
-            q2b = mma(pT_h, khTfl, q2b);
-            q3b = mma(pm_h, rhTfl, q3b);
-            q2 += q2b; q3 += q3b;
             const float tot_i = sm.tot[q][own], ent_i = sm.ent[q][own];
             float c[4], z[4];
 #pragma unroll
