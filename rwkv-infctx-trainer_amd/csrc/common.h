@@ -70,6 +70,16 @@ __device__ __forceinline__ float log_decay(float x, bool floor_decay, bool *floo
     return f ? LOG_W_FLOOR : l;
 }
 
+// The blocked kernels keep log w in base-2 units: -exp(x) log2(e) = -2^(x log2(e) + log2(log2(e))), so that
+// every later exponential is the bare hardware instruction.
+constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f, LOG2_LOG2E = 0.5287663729448977f;
+constexpr float LOG2_W_FLOOR = -7.643856189774724f;   // log2 0.005
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float log2_decay(float x, bool floor_decay) {
+    const float l = -exp2_fast(fmaf(x, LOG2E, LOG2_LOG2E));
+    return (floor_decay && l < LOG2_W_FLOOR) ? LOG2_W_FLOOR : l;
+}
+
 // ---- optional timing of one kernel with caller-owned HIP events (wkv_profile_events)
 enum KernelId {
     KID_NONE = 0, KID_REC_FORWARD = 1, KID_REC_BACKWARD = 2, KID_V4_FORWARD = 3, KID_V4_BACKWARD = 4,

@@ -210,6 +210,7 @@ __device__ __forceinline__ s4 frag_tr(const uint16_t *tile, int off) {
 //               inside the wavefront (two shuffles); the wavefront's total goes to `wtot` in LDS;
 //   scan_join   (at the start of the step, after that barrier): adds the totals of the earlier wavefronts of the
 //               block (inc = inclusive running sum inside the block) and forms the block total (tot).
+// All of these are in base-2 units (log2 w), so that every exponential is one v_exp_f32.
 __device__ __forceinline__ void scan_local(const float (&l)[4], float (&inc)[4], float (*wtot)[HEAD], int w16, int g, int n) {
 #pragma unroll
     for (int c = 0; c < 4; c++) {
@@ -223,14 +224,20 @@ __device__ __forceinline__ void scan_local(const float (&l)[4], float (&inc)[4],
     if (g == 3) *reinterpret_cast<float4 *>(&wtot[w16][4 * n]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
 }
 __device__ __forceinline__ void scan_join(float (&inc)[4], float (&tot)[4], const float (*wtot)[HEAD], int w16, int n) {
-    const int w0 = w16 & ~3, pos = w16 & 3;       // wavefront-uniform
-#pragma unroll
-    for (int c = 0; c < 4; c++) tot[c] = 0.f;
-#pragma unroll
-    for (int x = 0; x < 4; x++) {
-        const float4 t4 = *reinterpret_cast<const float4 *>(&wtot[w0 + x][4 * n]);
-        tot[0] += t4.x; tot[1] += t4.y; tot[2] += t4.z; tot[3] += t4.w;
-        if (x < pos) { inc[0] += t4.x; inc[1] += t4.y; inc[2] += t4.z; inc[3] += t4.w; }
+    const int w0 = w16 & ~3, pos = w16 & 3;       // wavefront-uniform: the branches below are scalar
+    const float4 t0 = *reinterpret_cast<const float4 *>(&wtot[w0][4 * n]), t1 = *reinterpret_cast<const float4 *>(&wtot[w0 + 1][4 * n]);
+    const float4 t2 = *reinterpret_cast<const float4 *>(&wtot[w0 + 2][4 * n]), t3 = *reinterpret_cast<const float4 *>(&wtot[w0 + 3][4 * n]);
+    const float a[4] = {t0.x + t1.x, t0.y + t1.y, t0.z + t1.z, t0.w + t1.w};
+    tot[0] = a[0] + (t2.x + t3.x); tot[1] = a[1] + (t2.y + t3.y); tot[2] = a[2] + (t2.z + t3.z); tot[3] = a[3] + (t2.w + t3.w);
+    if (pos == 1) {
+        inc[0] += t0.x; inc[1] += t0.y; inc[2] += t0.z; inc[3] += t0.w;
+        asm volatile("" ::: "memory");      // keeps the branch a branch (no select form with all the additions)
+    } else if (pos == 2) {
+        inc[0] += a[0]; inc[1] += a[1]; inc[2] += a[2]; inc[3] += a[3];
+        asm volatile("" ::: "memory");
+    } else if (pos == 3) {
+        inc[0] += a[0] + t2.x; inc[1] += a[1] + t2.y; inc[2] += a[2] + t2.z; inc[3] += a[3] + t2.w;
+        asm volatile("" ::: "memory");
     }
 }
 
@@ -278,8 +285,8 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
-        l_const = make_float4(log_decay(w4.x, floor_decay), log_decay(w4.y, floor_decay), log_decay(w4.z, floor_decay),
-                              log_decay(w4.w, floor_decay));
+        l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
+                              log2_decay(w4.w, floor_decay));
     }
     uint2 pa[4], pb[4];
     float4 pw[4];
@@ -309,7 +316,7 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int
                 const float lw4[4] = {pw[x].x, pw[x].y, pw[x].z, pw[x].w};
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
-                    l[x][c] = PER_TOKEN_W ? log_decay(lw4[c], floor_decay) : lw4[c];
+                    l[x][c] = PER_TOKEN_W ? log2_decay(lw4[c], floor_decay) : lw4[c];
                     run[c] += l[x][c];
                     inc[x][c] = run[c];
                 }
@@ -331,7 +338,7 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     const float ic = inc[x][c] + run[c];
-                    sc[c] = af[c] * __expf(BACKWARD ? ic - l[x][c] : tot[c] - ic);       // r e^{excl}  /  k e^{b-incl}
+                    sc[c] = af[c] * exp2_fast(BACKWARD ? ic - l[x][c] : tot[c] - ic);       // r e^{excl}  /  k e^{b-incl}
                 }
                 uint32_t h0, l0, h1, l1;
                 const int o = (tok0 + x) * LD + c4;
@@ -342,7 +349,7 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int
             }
             if (g == 3) {
                 *reinterpret_cast<float4 *>(&sm.tot[wv][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
-                *reinterpret_cast<float4 *>(&sm.dec[wv][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
+                *reinterpret_cast<float4 *>(&sm.dec[wv][c4]) = make_float4(exp2_fast(tot[0]), exp2_fast(tot[1]), exp2_fast(tot[2]), exp2_fast(tot[3]));
             }
         }
         lds_barrier();
@@ -367,7 +374,7 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int
     for (int kk = 0; kk < 4; kk++)
 #pragma unroll
         for (int e = 0; e < 4; e++) pp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = X[kk][e];
-    if (wv == 0) pp[HEAD * HEAD + lane] = __expf(dsum);
+    if (wv == 0) pp[HEAD * HEAD + lane] = exp2_fast(dsum);
 }
 
 template <bool PER_TOKEN_W>
@@ -403,8 +410,8 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
-        l_const = make_float4(log_decay(w4.x, floor_decay), log_decay(w4.y, floor_decay), log_decay(w4.z, floor_decay),
-                              log_decay(w4.w, floor_decay));
+        l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
+                              log2_decay(w4.w, floor_decay));
     }
     uint2 pr, pk, pv;
     float4 pw;
@@ -433,7 +440,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
         lc[0] = pw.x; lc[1] = pw.y; lc[2] = pw.z; lc[3] = pw.w;
         if (PER_TOKEN_W) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) lc[c] = log_decay(lc[c], floor_decay);
+            for (int c = 0; c < 4; c++) lc[c] = log2_decay(lc[c], floor_decay);
         }
         scan_local(lc, ic, sm.wtot, w16, g, n);
     };
@@ -457,8 +464,8 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             float rhv[4], khv[4], p = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                rhv[c] = rf[c] * __expf(inc[c] - l[c]);
-                khv[c] = kf[c] * __expf(tot[c] - inc[c]);
+                rhv[c] = rf[c] * exp2_fast(inc[c] - l[c]);
+                khv[c] = kf[c] * exp2_fast(tot[c] - inc[c]);
                 p = fmaf(rf[c] * uf[c], kf[c], p);
             }
             uint32_t h0, l0, h1, l1;
@@ -472,8 +479,8 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
             *reinterpret_cast<uint2 *>(&sm.v[ot]) = pv;
             if ((w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
                 if (g == 3) {
-                    *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
-                    *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(__expf(-tot[0]), __expf(-tot[1]), __expf(-tot[2]), __expf(-tot[3]));
+                    *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(exp2_fast(tot[0]), exp2_fast(tot[1]), exp2_fast(tot[2]), exp2_fast(tot[3]));
+                    *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(exp2_fast(-tot[0]), exp2_fast(-tot[1]), exp2_fast(-tot[2]), exp2_fast(-tot[3]));
                 }
             }
             p = row_prefix_sum(p);           // lane 15 of the row ends with the sum over the 64 channels
@@ -716,8 +723,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
         const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
-        l_const = make_float4(log_decay(w4.x, floor_decay), log_decay(w4.y, floor_decay), log_decay(w4.z, floor_decay),
-                              log_decay(w4.w, floor_decay));
+        l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
+                              log2_decay(w4.w, floor_decay));
     }
     uint2 pr, pk, pv, pg;
     float4 pw;
@@ -773,7 +780,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
             if (PER_TOKEN_W) {
 #pragma unroll
-                for (int c = 0; c < 4; c++) l[c] = log_decay(l[c], floor_decay);
+                for (int c = 0; c < 4; c++) l[c] = log2_decay(l[c], floor_decay);
             }
             if (have_out) write_out(sb + 1, tok, c4);
             scan_local(l, inc, sm.wtot, w16, g, n);      // (the one-step-ahead form of forward16 costs registers this kernel lacks)
@@ -782,8 +789,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             float rhv[4], khv[4], p = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                rhv[c] = rf[c] * __expf(inc[c] - l[c]);
-                khv[c] = kf[c] * __expf(tot[c] - inc[c]);
+                rhv[c] = rf[c] * exp2_fast(inc[c] - l[c]);
+                khv[c] = kf[c] * exp2_fast(tot[c] - inc[c]);
                 p = fmaf(rf[c] * uf[c], kf[c], p);
             }
             uint32_t h0, l0, h1, l1;
@@ -804,8 +811,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             if ((w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
                 if (g == 3) {
                     *reinterpret_cast<float4 *>(&sm.tot[q][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
-                    *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(__expf(tot[0]), __expf(tot[1]), __expf(tot[2]), __expf(tot[3]));
-                    *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(__expf(-tot[0]), __expf(-tot[1]), __expf(-tot[2]), __expf(-tot[3]));
+                    *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(exp2_fast(tot[0]), exp2_fast(tot[1]), exp2_fast(tot[2]), exp2_fast(tot[3]));
+                    *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(exp2_fast(-tot[0]), exp2_fast(-tot[1]), exp2_fast(-tot[2]), exp2_fast(-tot[3]));
                 }
             }
             p = row_prefix_sum(p);           // lane 15 of the row ends with the sum over the 64 channels
@@ -994,7 +1001,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
             for (int e = 0; e < 4; e++) {
                 const int tk = 16 * q + 4 * g + e;
                 const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
-                const float E1 = __expf(exc), E2 = __expf(tot_i - inc);
+                const float E1 = exp2_fast(exc), E2 = exp2_fast(tot_i - inc);
                 const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
                 const uint32_t rkv = sm.rk[tk * HEAD + own];
                 const float rr = bf_lo(rkv), kr = bf_hi(rkv);
@@ -1003,7 +1010,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
                 const float gkv = gkn + u_i * rr * pd;
                 c[e] = rr * grv - kr * gkv;
                 z[e] = kr * gkn;
-                lfac[e] = (floor_decay && l <= LOG_W_FLOOR) ? 0.f : l;
+                lfac[e] = (floor_decay && l <= LOG2_W_FLOOR) ? 0.f : l * LN2;       // back to the natural logarithm
                 gu_acc = fmaf(rr * kr, pd, gu_acc);
                 // this wavefront was the only reader left of its (block, quarter) corner of the rh and kh tiles
                 sm.rh[tk * LD + own] = bf16_bits(grv);
