@@ -9,6 +9,12 @@ is one forward + one backward call through the C ABI with all inputs resident
 in HBM.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--cfg 1|2|3|4] [--algo auto|recurrent|chunked]
+                    [--launch graph|eager]
+
+The K timed steps are launched from a HIP graph that holds one period of the
+input rotation (six steps; what is left of K after whole replays runs as plain
+launches), or as plain launches throughout with ``--launch eager`` (and whenever
+the capture fails).
 """
 import argparse
 import ctypes
@@ -35,6 +41,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline times")
     ap.add_argument("--rotate", type=int, default=3, help="distinct input sets cycled through")
+    ap.add_argument("--launch", default="graph", choices=["graph", "eager"],
+                    help="timed steps replayed from a HIP graph of one rotation period, or launched one by one")
     ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run three plain 256 MiB device copies first (reference point for the FETCH_SIZE / "
@@ -154,6 +162,32 @@ class Runner4:
         return {"forward": (3,), "backward": (4,)}
 
 
+def capture_period(runner, period):
+    """One period of steps (input rotation x state ping-pong) recorded into a HIP graph.
+    The library allocates nothing and synchronises nothing in a call, so its launches
+    record as they are.  Returns None when the capture fails."""
+    torch = runner.torch
+    assert runner.i % period == 0
+    eager_stream, i0 = runner.stream, runner.i
+    try:
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                runner.stream = torch.cuda.current_stream().cuda_stream
+                for _ in range(period):
+                    runner.step()
+        torch.cuda.current_stream().wait_stream(side)
+        return g
+    except Exception as e:            # noqa: BLE001 - any capture problem means plain launches
+        print(f"bench.py: HIP graph capture failed ({e}); timing plain launches", file=sys.stderr)
+        runner.i = i0
+        return None
+    finally:
+        runner.stream = eager_stream
+
+
 def time_kernel(runner, kid, steps):
     """Average launch duration (ms) of kernel `kid` over `steps` steps, by HIP
     events recorded inside the library on the launch stream."""
@@ -249,12 +283,23 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-    for _ in range(a.warmup):
+    period = 2 * a.rotate if a.rotate % 2 else a.rotate        # input rotation x state ping-pong
+    for _ in range(-(-max(a.warmup, 1) // period) * period if a.launch == "graph" else a.warmup):
         runner.step()
     torch.cuda.synchronize()
+    graph = capture_period(runner, period) if a.launch == "graph" else None
+    if graph is not None:
+        graph.replay()                 # untimed: the first replay uploads the graph
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(a.steps):
-        runner.step()
+    if graph is not None:
+        for _ in range(a.steps // period):
+            graph.replay()
+        for _ in range(a.steps % period):
+            runner.step()
+    else:
+        for _ in range(a.steps):
+            runner.step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_step = dt / a.steps * 1e3
@@ -285,7 +330,8 @@ def main():
            "value": tok_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": runner.dtype_name, "data": "synthetic",
-           "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto"},
+           "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto",
+                      "launch": f"hip graph of {period} steps per replay" if graph is not None else "eager"},
            "roofline": roofline}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(a.cfg, a.cpu_heads)
