@@ -413,19 +413,20 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
         l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
                               log2_decay(w4.w, floor_decay));
     }
-    uint2 pr, pk, pv;
-    float4 pw;
-    auto fetch = [&](int sb) {
+    // the inputs of this lane's token, fetched two steps ahead into two register sets used in turn
+    struct Row { uint2 r, k, v; float4 w; };
+    Row rowA, rowB;
+    auto fetch = [&](int sb, Row &x) __attribute__((always_inline)) {
         const int t = sb * SB + tok;
         if (t < Tlen) {
             const size_t o = base + (size_t)t * C + c4;
-            pr = *reinterpret_cast<const uint2 *>(r + o);
-            pk = *reinterpret_cast<const uint2 *>(k + o);
-            pv = *reinterpret_cast<const uint2 *>(v + o);
-            pw = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+            x.r = *reinterpret_cast<const uint2 *>(r + o);
+            x.k = *reinterpret_cast<const uint2 *>(k + o);
+            x.v = *reinterpret_cast<const uint2 *>(v + o);
+            x.w = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
         } else {
-            pr = pk = pv = make_uint2(0u, 0u);
-            pw = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+            x.r = x.k = x.v = make_uint2(0u, 0u);
+            x.w = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
     const int tro = tr_lane_offset(lane, LDT);
@@ -433,10 +434,11 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
     const size_t ck_off = (size_t)bh * (nsb + 1) * HEAD * HEAD;
 
     bool have_y = false;
-    fetch(sb0);
+    fetch(sb0, rowA);
+    if (sb0 + 1 < sb1) fetch(sb0 + 1, rowB);
     // log w of this lane's token and its running sum inside the wavefront, always one step ahead (see scan_local)
     float lc[4], ic[4];
-    auto scan_ahead = [&]() {
+    auto scan_ahead = [&](const float4 &pw) __attribute__((always_inline)) {
         lc[0] = pw.x; lc[1] = pw.y; lc[2] = pw.z; lc[3] = pw.w;
         if (PER_TOKEN_W) {
 #pragma unroll
@@ -444,10 +446,12 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
         }
         scan_local(lc, ic, sm.wtot, w16, g, n);
     };
-    scan_ahead();
+    scan_ahead(rowA.w);
     lds_barrier();
     PT_DECL
-    for (int sb = sb0; sb < sb1; sb++) {
+    // one step; `cur` holds its inputs (and takes those of the step after the next), `nxt` those of the next step
+    auto do_step = [&](const int sb, Row &cur, const Row &nxt) __attribute__((always_inline)) {
+        const uint2 pr = cur.r, pk = cur.k, pv = cur.v;
         PT_MARK(5)
         // ---------------- prepare the scaled operands of this lane's token
         {
@@ -489,7 +493,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
         PT_MARK(0)
         lds_barrier();
         PT_MARK(1)
-        if (sb + 1 < sb1) fetch(sb + 1);          // next step's loads fly during the MFMA phase
+        if (sb + 2 < sb1) fetch(sb + 2, cur);     // these loads have two steps to arrive
 
         if (chain) {
             if (ckpt) {       // state at the start of this step, 16 bytes per lane and tile
@@ -564,10 +568,14 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
 #pragma unroll
             for (int e = 0; e < 4; e++) sm.rh[(16 * q + 4 * g + e) * LD + 16 * wv + n] = bf16_bits(yt[e]);
         }
-        if (sb + 1 < sb1) scan_ahead();      // the next step's w has arrived by now
+        if (sb + 1 < sb1) scan_ahead(nxt.w);
         PT_MARK(4)
         lds_barrier();
         have_y = y != nullptr;
+    };
+    for (int sb = sb0; sb < sb1; sb += 2) {
+        do_step(sb, rowA, rowB);
+        if (sb + 1 < sb1) do_step(sb + 1, rowB, rowA);
     }
     if (have_y) {
         const int t = (sb1 - 1) * SB + tok;
