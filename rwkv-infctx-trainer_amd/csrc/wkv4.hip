@@ -26,22 +26,34 @@ constexpr float NEG_HUGE = -1e38f;
 
 struct Chain { float p, q, o, dp, dq; };
 
-// one token: output y and the pieces backward re-uses; advances the chain
+// Two terms scaled by a common maximum exponent, e^{a-m} and e^{b-m} with m = max(a, b): one of the two is
+// exactly 1, so a pair costs one exponential, e^{-|a-b|}.
+struct ExpPair { float first, second; bool first_is_max; };
+__device__ __forceinline__ ExpPair exp_pair(float a, float b) {
+    const float d = a - b, e = __expf(-fabsf(d));
+    const bool fm = d >= 0.f;
+    return ExpPair{fm ? 1.f : e, fm ? e : 1.f, fm};
+}
+
+// one token: output y and the pieces backward re-uses (1 / scaled denominator, the current token's scaled weight,
+// the history's scaled weight, minus the scaling exponent); advances the chain
 __device__ __forceinline__ float v4_step(Chain &s, float w, float u, float kk, float vv,
-                                         float &iden, float &cexp, float &hist_w) {
-    const float m = fmaxf(s.o, u + kk);
-    hist_w = __expf(s.o - m);
-    cexp = u + kk - m;
-    const float ec = __expf(cexp);
-    iden = __frcp_rn(hist_w * s.q + ec);
+                                         float &iden, float &ec, float &hist_w, float &neg_m) {
+    const float uk = u + kk;
+    const ExpPair a = exp_pair(s.o, uk);
+    hist_w = a.first;
+    ec = a.second;
+    neg_m = a.first_is_max ? -s.o : -uk;
+    iden = __builtin_amdgcn_rcpf(hist_w * s.q + ec);      // the bare v_rcp_f32 (1 ulp), not a full division
     const float y = (hist_w * s.p + ec * vv) * iden;
-    const float m2 = fmaxf(w + s.o, kk);
-    const float dh = __expf(w + s.o - m2), dc = __expf(kk - m2);
+    const float wo = w + s.o;
+    const ExpPair d = exp_pair(wo, kk);
+    const float dh = d.first, dc = d.second;
     s.dp = dh * (s.p + s.dp);
     s.dq = dh * (s.q + s.dq);
     s.p = fmaf(dh, s.p, dc * vv);
     s.q = fmaf(dh, s.q, dc);
-    s.o = m2;
+    s.o = d.first_is_max ? wo : kk;
     return y;
 }
 
@@ -90,24 +102,25 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
                 float *cp = ckpt + (size_t)blk * 5 * BC + idx;
                 cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
             }
-            T *yp = y ? y + base + (size_t)t0 * C : nullptr;
             const int cnt = min(CK, Tlen - t0);
-            if (cnt == CK) {
+            // (y or no y, whole block or not: decided once per block, so that the 16 tokens are straight-line code)
+            auto tokens = [&](auto with_y, auto full) {
+                T *yp = y + base + (size_t)t0 * C;
 #pragma unroll
                 for (int i = 0; i < CK; i++) {
-                    float iden, cexp, hw;
-                    const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, cexp, hw);
-                    if (yp) { *yp = from_float<T>(yy); yp += C; }
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < CK; i++) {
-                    if (i < cnt) {
-                        float iden, cexp, hw;
-                        const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, cexp, hw);
-                        if (yp) { *yp = from_float<T>(yy); yp += C; }
+                    if (decltype(full)::value || i < cnt) {
+                        float iden, ec, hw, nm;
+                        const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, ec, hw, nm);
+                        if (decltype(with_y)::value) { *yp = from_float<T>(yy); yp += C; }
                     }
                 }
+            };
+            if (y) {
+                if (cnt == CK) tokens(std::true_type{}, std::true_type{});
+                else tokens(std::true_type{}, std::false_type{});
+            } else {
+                if (cnt == CK) tokens(std::false_type{}, std::true_type{});
+                else tokens(std::false_type{}, std::false_type{});
             }
             if (t0 + RING * CK < Tlen) fetch(t0 + RING * CK, bk[d], bv[d]);
         }
@@ -157,15 +170,15 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
     auto block = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain s) {
         constexpr bool FULL = decltype(full_tag)::value;
         const int t0 = blk * CK, cnt = FULL ? CK : Tlen - t0;
-        float ys[CK], iden[CK], cexp[CK];
+        float ys[CK], iden[CK], ec[CK], neg_m[CK];
 #pragma unroll
         for (int i = 0; i < CK; i++) {
             if (FULL || i < cnt) {
                 const float dp0 = s.dp, dq0 = s.dq;
                 float hw;
-                ys[i] = v4_step(s, w, u, kk[i], vv[i], iden[i], cexp[i], hw);
+                ys[i] = v4_step(s, w, u, kk[i], vv[i], iden[i], ec[i], hw, neg_m[i]);
                 acc_w += gg[i] * (dp0 - dq0 * ys[i]) * iden[i] * hw;
-                acc_u += gg[i] * (vv[i] - ys[i]) * __expf(cexp[i]) * iden[i];
+                acc_u += gg[i] * (vv[i] - ys[i]) * ec[i] * iden[i];
             }
         }
         if (blk == nblk - 1 && gs_out) {       // gradient arriving through the state handed out
@@ -178,17 +191,16 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
 #pragma unroll
         for (int i = CK - 1; i >= 0; i--, gkp -= C, gvp -= C) {
             if (FULL || i < cnt) {
-                const float direct = gg[i] * iden[i] * __expf(cexp[i]);
+                const float direct = gg[i] * iden[i] * ec[i];
                 const float later = __expf(kk[i] + go);
                 *gkp = from_float<T>(direct * (vv[i] - ys[i]) + later * (gp * vv[i] + gq));
                 *gvp = from_float<T>(direct + later * gp);
-                const float hist = cexp[i] - kk[i] - u;
-                const float m = fmaxf(w + go, hist);
-                const float keep = __expf(w + go - m);
-                const float add = gg[i] * iden[i] * __expf(hist - m);
-                gp = fmaf(keep, gp, add);
-                gq = fmaf(keep, gq, -add * ys[i]);
-                go = m;
+                const float wg = w + go;
+                const ExpPair e = exp_pair(wg, neg_m[i]);      // gy_t / den_t carries the exponent -m_t
+                const float add = gg[i] * iden[i] * e.second;
+                gp = fmaf(e.first, gp, add);
+                gq = fmaf(e.first, gq, -add * ys[i]);
+                go = e.first_is_max ? wg : neg_m[i];
             }
         }
     };
