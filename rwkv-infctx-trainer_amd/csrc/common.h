@@ -80,6 +80,12 @@ __device__ __forceinline__ float log2_decay(float x, bool floor_decay) {
     return (floor_decay && l < LOG2_W_FLOOR) ? LOG2_W_FLOOR : l;
 }
 
+// Workgroup barrier that waits for this wavefront's LDS traffic only: __syncthreads() would also wait for every
+// global load in flight, i.e. for the prefetch the barrier is meant to overlap with.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- optional timing of one kernel with caller-owned HIP events (wkv_profile_events)
 enum KernelId {
     KID_NONE = 0, KID_REC_FORWARD = 1, KID_REC_BACKWARD = 2, KID_V4_FORWARD = 3, KID_V4_BACKWARD = 4,

@@ -1,11 +1,13 @@
 // RWKV-v4 WKV with (aa, bb, pp) state: one lane per (batch, channel) chain.
 //
-// The chain is serial in time, so the kernels keep many independent loads in
-// flight per lane instead: blocks of 16 tokens of k, v (and gy) are fetched
-// into registers two (backward: one) blocks ahead of the one being consumed;
-// consecutive lanes are consecutive channels, so every load and store is a full
-// coalesced row.  The speed is set by one wavefront's walk over T (about 450
-// cycles per token forward): partly filled wavefronts on more SIMDs do not help.
+// The chain is serial in time, and a GPU holds few chains (B*C lanes: one or two
+// wavefronts per CU), so what sets the speed is how many bytes each lane keeps
+// in flight: blocks of 16 tokens of k, v (and gy) are fetched into registers
+// three blocks ahead of the one being consumed; consecutive lanes are consecutive
+// channels, so every load and store is a full coalesced row.  Per token the
+// arithmetic is kept short (one exponential per max-scaled pair, the bare
+// reciprocal instruction) and free of branches, so that the tokens of a block are
+// one straight-line stretch the scheduler can interleave.
 //
 // State convention (RWKV-v4neo/cuda/wkv_cuda_bf16.cu:30-52): (p, q, o) with
 // p, q the decayed sums divided by e^{o}.  Backward carries the state gradient
@@ -15,7 +17,8 @@
 // Backward never stores per-token intermediates for the whole sequence (the
 // reference keeps three T-long arrays per lane): the forward sweep leaves a
 // 5-float checkpoint (p, q, o, dp/dw, dq/dw) every 16 tokens, and the backward
-// sweep replays one 16-token block at a time from its checkpoint.
+// sweep replays one 16-token block at a time from its checkpoint (a second
+// wavefront walks the block replayed just before backwards at the same time).
 #include "common.h"
 #include <type_traits>
 
@@ -72,9 +75,8 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
     Chain s{0.f, 0.f, NEG_HUGE, 0.f, 0.f};
     if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
 
-    // three 16-token blocks of k, v per lane: one being consumed, two in flight (a chain is serial and a CU holds
-    // few chains, so the bytes in flight per lane are what sets the bandwidth); indexed statically by unrolling
-    constexpr int RING = 3;
+    // RING 16-token blocks of k, v per lane: one being consumed, the others in flight; indexed statically by unrolling
+    constexpr int RING = 4;
     float bk[RING][CK], bv[RING][CK];
     auto fetch = [&](int t0, float (&kk)[CK], float (&vv)[CK]) {
         const T *kp = k + base + (size_t)t0 * C, *vp = v + base + (size_t)t0 * C;
@@ -128,26 +130,34 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
     if (s_out) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
 }
 
+// Backward: two wavefronts per 64 chains.  Replaying a block from its checkpoint does not depend on the reverse
+// walk of the blocks after it, so the two halves of the work run side by side: wavefront 0 replays block b (and
+// sums the decay / bonus gradients), leaving y, 1/denominator, the current token's weight and the scaling exponent
+// of its 16 tokens in LDS; wavefront 1 meanwhile walks block b+1 backwards from what wavefront 0 left the step
+// before.  One workgroup barrier per block; RB LDS buffers and RB register sets of inputs (one being consumed,
+// the others in flight) used in turn.
+constexpr int RB = 4;
+struct V4Replay { float ys[CK][64], iden[CK][64], ec[CK][64], neg_m[CK][64]; };
+
 template <class T>
-__global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
+__global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
         const float *__restrict__ time_first, const T *__restrict__ k, const T *__restrict__ v,
         const T *__restrict__ gy, const float *__restrict__ gs_out, const float *__restrict__ ckpt,
         float *__restrict__ gw_part, float *__restrict__ gu_part, T *__restrict__ gk, T *__restrict__ gv,
         float *__restrict__ gs_in)
 {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= BC) return;
+    __shared__ V4Replay sh[RB];
+    const int lane = threadIdx.x & 63, role = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int idx = blockIdx.x * 64 + lane;
+    if (idx >= BC) return;          // (the same lanes leave in both wavefronts; the barriers count wavefronts)
     const int b = idx / C, c = idx % C;
     const float w = -__expf(time_decay[c]), u = time_first[c];
     const size_t base = (size_t)b * Tlen * C + c;
-
-    float gp = 0.f, gq = 0.f, go = NEG_HUGE, acc_w = 0.f, acc_u = 0.f;
     const int nblk = (Tlen + CK - 1) / CK;
-    // two blocks of k, v, gy and their checkpoints per lane: one being consumed, one in flight
-    constexpr int RING = 2;
-    float bk[RING][CK], bv[RING][CK], bg[RING][CK];
-    Chain bs[RING];
-    auto fetch = [&](int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain &cs) {
+
+    // RB blocks of k, v, gy per lane: one being consumed, the others in flight
+    float bk[RB][CK], bv[RB][CK], bg[RB][CK];
+    auto fetch = [&](int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK]) {
         const int t0 = blk * CK;
         const size_t o0 = base + (size_t)t0 * C;
         const T *kp = k + o0, *vp = v + o0, *gp_ = gy + o0;
@@ -163,63 +173,106 @@ __global__ __launch_bounds__(64) void v4_backward(int BC, int Tlen, int C, const
                 gg[i] = in ? to_float(*gp_) : 0.f;
             }
         }
-        const float *cp = ckpt + (size_t)blk * 5 * BC + idx;
-        cs = Chain{cp[0], cp[BC], cp[2 * (size_t)BC], cp[3 * (size_t)BC], cp[4 * (size_t)BC]};
     };
-    // one block: replay it forward from its checkpoint, then walk it backwards (FULL: all CK tokens exist)
-    auto block = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain s) {
-        constexpr bool FULL = decltype(full_tag)::value;
-        const int t0 = blk * CK, cnt = FULL ? CK : Tlen - t0;
-        float ys[CK], iden[CK], ec[CK], neg_m[CK];
+    auto load_ckpt = [&](int blk) {
+        const float *cp = ckpt + (size_t)blk * 5 * BC + idx;
+        return Chain{cp[0], cp[BC], cp[2 * (size_t)BC], cp[3 * (size_t)BC], cp[4 * (size_t)BC]};
+    };
+
+    if (role == 0) {
+        // ---------------- replay: step j handles block nblk-1-j, register set and LDS buffer j % RB
+        float acc_w = 0.f, acc_u = 0.f;
+        Chain bs[RB];
 #pragma unroll
-        for (int i = 0; i < CK; i++) {
-            if (FULL || i < cnt) {
-                const float dp0 = s.dp, dq0 = s.dq;
-                float hw;
-                ys[i] = v4_step(s, w, u, kk[i], vv[i], iden[i], ec[i], hw, neg_m[i]);
-                acc_w += gg[i] * (dp0 - dq0 * ys[i]) * iden[i] * hw;
-                acc_u += gg[i] * (vv[i] - ys[i]) * ec[i] * iden[i];
+        for (int d = 0; d < RB; d++)
+            if (nblk - 1 - d >= 0) { fetch(nblk - 1 - d, bk[d], bv[d], bg[d]); bs[d] = load_ckpt(nblk - 1 - d); }
+        auto replay = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain s, V4Replay &out) {
+            constexpr bool FULL = decltype(full_tag)::value;
+            const int cnt = FULL ? CK : Tlen - blk * CK;
+#pragma unroll
+            for (int i = 0; i < CK; i++) {
+                if (FULL || i < cnt) {
+                    const float dp0 = s.dp, dq0 = s.dq;
+                    float hw, iden, ec, nm;
+                    const float yy = v4_step(s, w, u, kk[i], vv[i], iden, ec, hw, nm);
+                    acc_w += gg[i] * (dp0 - dq0 * yy) * iden * hw;
+                    acc_u += gg[i] * (vv[i] - yy) * ec * iden;
+                    out.ys[i][lane] = yy; out.iden[i][lane] = iden; out.ec[i][lane] = ec; out.neg_m[i][lane] = nm;
+                }
             }
+            if (blk == nblk - 1 && gs_out) {       // gradient arriving through the state handed out
+                const float gp = gs_out[idx * 3], gq = gs_out[idx * 3 + 1];
+                const float go = (gp == 0.f && gq == 0.f) ? NEG_HUGE : gs_out[idx * 3 + 2];
+                acc_w += (gp * s.dp + gq * s.dq) * __expf(s.o + go);
+            }
+        };
+        auto step = [&](int j, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain &cs, V4Replay &out) {
+            const int blk = nblk - 1 - j;
+            if (blk >= 0) {
+                if ((blk + 1) * CK <= Tlen) replay(std::true_type{}, blk, kk, vv, gg, cs, out);
+                else replay(std::false_type{}, blk, kk, vv, gg, cs, out);
+                if (blk - RB >= 0) { fetch(blk - RB, kk, vv, gg); cs = load_ckpt(blk - RB); }
+            }
+            lds_barrier();
+        };
+        for (int j = 0; j <= nblk; j += RB) {
+#pragma unroll
+            for (int d = 0; d < RB; d++)
+                if (j + d <= nblk) step(j + d, bk[d], bv[d], bg[d], bs[d], sh[d]);
         }
-        if (blk == nblk - 1 && gs_out) {       // gradient arriving through the state handed out
+        gw_part[idx] = acc_w * w;
+        gu_part[idx] = acc_u;
+    } else {
+        // ---------------- reverse walk: step j handles block nblk-j (none at j = 0), register set and buffer (j-1) % RB
+        float gp = 0.f, gq = 0.f, go = NEG_HUGE;
+        if (gs_out) {
             gp = gs_out[idx * 3]; gq = gs_out[idx * 3 + 1]; go = gs_out[idx * 3 + 2];
             if (gp == 0.f && gq == 0.f) go = NEG_HUGE;
-            acc_w += (gp * s.dp + gq * s.dq) * __expf(s.o + go);
         }
-        const size_t oe = base + (size_t)(t0 + CK - 1) * C;
-        T *gkp = gk + oe, *gvp = gv + oe;
 #pragma unroll
-        for (int i = CK - 1; i >= 0; i--, gkp -= C, gvp -= C) {
-            if (FULL || i < cnt) {
-                const float direct = gg[i] * iden[i] * ec[i];
-                const float later = __expf(kk[i] + go);
-                *gkp = from_float<T>(direct * (vv[i] - ys[i]) + later * (gp * vv[i] + gq));
-                *gvp = from_float<T>(direct + later * gp);
-                const float wg = w + go;
-                const ExpPair e = exp_pair(wg, neg_m[i]);      // gy_t / den_t carries the exponent -m_t
-                const float add = gg[i] * iden[i] * e.second;
-                gp = fmaf(e.first, gp, add);
-                gq = fmaf(e.first, gq, -add * ys[i]);
-                go = e.first_is_max ? wg : neg_m[i];
+        for (int d = 0; d < RB; d++)
+            if (nblk - 1 - d >= 0) fetch(nblk - 1 - d, bk[d], bv[d], bg[d]);
+        auto walk = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], const V4Replay &in) {
+            constexpr bool FULL = decltype(full_tag)::value;
+            const int t0 = blk * CK, cnt = FULL ? CK : Tlen - t0;
+            const size_t oe = base + (size_t)(t0 + CK - 1) * C;
+            T *gkp = gk + oe, *gvp = gv + oe;
+#pragma unroll
+            for (int i = CK - 1; i >= 0; i--, gkp -= C, gvp -= C) {
+                if (FULL || i < cnt) {
+                    const float ys = in.ys[i][lane], iden = in.iden[i][lane], ec = in.ec[i][lane], nm = in.neg_m[i][lane];
+                    const float direct = gg[i] * iden * ec;
+                    const float later = __expf(kk[i] + go);
+                    *gkp = from_float<T>(direct * (vv[i] - ys) + later * (gp * vv[i] + gq));
+                    *gvp = from_float<T>(direct + later * gp);
+                    const float wg = w + go;
+                    const ExpPair e = exp_pair(wg, nm);      // gy_t / den_t carries the exponent -m_t
+                    const float add = gg[i] * iden * e.second;
+                    gp = fmaf(e.first, gp, add);
+                    gq = fmaf(e.first, gq, -add * ys);
+                    go = e.first_is_max ? wg : nm;
+                }
+            }
+        };
+        auto step = [&](int j, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], const V4Replay &in) {
+            const int blk = nblk - j;
+            if (j >= 1) {
+                if ((blk + 1) * CK <= Tlen) walk(std::true_type{}, blk, kk, vv, gg, in);
+                else walk(std::false_type{}, blk, kk, vv, gg, in);
+                if (blk - RB >= 0) fetch(blk - RB, kk, vv, gg);
+            }
+            lds_barrier();
+        };
+        for (int j = 0; j <= nblk; j += RB) {
+#pragma unroll
+            for (int d = 0; d < RB; d++) {
+                constexpr int dummy = 0; (void)dummy;
+                const int e = (d + RB - 1) % RB;
+                if (j + d <= nblk) step(j + d, bk[e], bv[e], bg[e], sh[e]);
             }
         }
-    };
-#pragma unroll
-    for (int d = 0; d < RING; d++)
-        if (nblk - 1 - d >= 0) fetch(nblk - 1 - d, bk[d], bv[d], bg[d], bs[d]);
-    for (int bb = nblk - 1; bb >= 0; bb -= RING) {
-#pragma unroll
-        for (int d = 0; d < RING; d++) {
-            const int blk = bb - d;
-            if (blk < 0) break;
-            if ((blk + 1) * CK <= Tlen) block(std::true_type{}, blk, bk[d], bv[d], bg[d], bs[d]);
-            else block(std::false_type{}, blk, bk[d], bv[d], bg[d], bs[d]);
-            if (blk - RING >= 0) fetch(blk - RING, bk[d], bv[d], bg[d], bs[d]);
-        }
+        if (gs_in) { gs_in[idx * 3] = gp; gs_in[idx * 3 + 1] = gq; gs_in[idx * 3 + 2] = go; }
     }
-    if (gs_in) { gs_in[idx * 3] = gp; gs_in[idx * 3 + 1] = gq; gs_in[idx * 3 + 2] = go; }
-    gw_part[idx] = acc_w * w;
-    gu_part[idx] = acc_u;
 }
 
 size_t v4_checkpoint_bytes(int B, int Tlen, int C) {
@@ -252,7 +305,7 @@ static hipError_t bwd(hipStream_t s, int B, int Tlen, int C, const float *td, co
         ckpt = own_ckpt;
     }
     prof_begin(KID_V4_BACKWARD, s);
-    hipLaunchKernelGGL((v4_backward<T>), dim3((BC + 63) / 64), dim3(64), 0, s, BC, Tlen, C, td, tf, (const T *)k,
+    hipLaunchKernelGGL((v4_backward<T>), dim3((BC + 63) / 64), dim3(128), 0, s, BC, Tlen, C, td, tf, (const T *)k,
                        (const T *)v, (const T *)gy, gs_out, ckpt, gw_part, gu_part, (T *)gk, (T *)gv, gs_in);
     prof_end(KID_V4_BACKWARD, s);
     hipError_t e = hipGetLastError();

@@ -54,12 +54,7 @@ namespace chunked {
 #define PT_PRINT(name)
 #endif
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
-// outstanding global load, which would stall each phase on the prefetch of the next step;
-// the wavefronts of these kernels talk to each other through LDS alone.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
+// (lds_barrier(): the workgroup barrier of these kernels, whose wavefronts talk to each other through LDS alone)
 
 typedef short s4 __attribute__((ext_vector_type(4)));
 typedef short s8 __attribute__((ext_vector_type(8)));
