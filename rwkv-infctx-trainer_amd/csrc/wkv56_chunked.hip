@@ -257,13 +257,13 @@ struct PassTiles {
 };
 
 template <bool PER_TOKEN_W, bool BACKWARD>
-__global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int nseg, int sps, int m, int pps,
+__global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, int H, int nseg, int sps, int m, int pps,
         const bf16 *__restrict__ a_in, const bf16 *__restrict__ b_in, const float *__restrict__ wraw,
         float *__restrict__ part, int floor_decay)
 {
     __shared__ __align__(16) PassTiles sm;
     const int units = (nseg - 1) * m;       // workgroups per (batch, head)
-    const int bh = blockIdx.x / units, piece = (BACKWARD ? m : 0) + blockIdx.x % units, seg = piece / m, b = bh / H, h = bh % H;
+    const int bh = bh0 + blockIdx.x / units, piece = (BACKWARD ? m : 0) + blockIdx.x % units, seg = piece / m, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
@@ -373,7 +373,7 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int Tlen, int C, int H, int
 }
 
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int nseg, int sps, int m,
+__global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
         bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, const float *__restrict__ part,
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int Tlen, int C, int H, int 
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Fwd16Tiles &sm = *reinterpret_cast<Fwd16Tiles *>(smem_raw);
-    const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
+    const int bh = bh0 + blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
     const int q = w16 >> 2, wv = w16 & 3;          // block and quarter for preparing and finishing
     const bool chain = w16 < 8, builder = w16 >= 8 && w16 < 12;
@@ -667,7 +667,7 @@ constexpr int NT_B16 = 1024;
     (void)tro; (void)c4; (void)tok; (void)own;
 
 template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int nseg, int sps, int m,
+__global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
         const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
@@ -676,7 +676,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Bwd16Tiles &sm = *reinterpret_cast<Bwd16Tiles *>(smem_raw);
-    const int bh = blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
+    const int bh = bh0 + blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
     const int role = w16 >> 2, q = role, wv = w16 & 3;      // chain role; block (for preparing and for the block phase); quarter
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
@@ -1080,16 +1080,33 @@ __global__ __launch_bounds__(NT_B16) void backward16(int Tlen, int C, int H, int
     }
 }
 
+// Sums the per-(batch, segment) partial sums of gu (gw) in a fixed order.  The (batch, head) pairs below nA ran as
+// one segment and left theirs in `one` [b][C]; the others ran as nseg segments and left theirs in `many`
+// [(b*nseg + seg)][C].
+__global__ void sum_partials(int B, int H, int nA, int nseg, const float *__restrict__ one, const float *__restrict__ many,
+                             float *__restrict__ out) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, C = H * HEAD;
+    if (c >= C) return;
+    const int h = c / HEAD;
+    float sum = 0.f;
+    for (int b = 0; b < B; b++) {
+        if (b * H + h < nA) sum += one[(size_t)b * C + c];
+        else
+            for (int x = 0; x < nseg; x++) sum += many[(size_t)(b * nseg + x) * C + c];
+    }
+    out[c] = sum;
+}
+
 // Chains the piece summaries (S_out = decay o S_in + delta, one decay per key) of one
 // (batch, head) in order, one lane per state element.  `first`..`last` are the pieces
 // the pass produced; going up (forward, step = +1) it starts from `start` and leaves
 // the state at the start of segment s in the slot of piece s*m - 1; going down
 // (backward, step = -1) it leaves the gradient at the end of segment s in the slot of
 // piece (s+1)*m.  In place: a slot is overwritten by the lane that has just read it.
-__global__ __launch_bounds__(256) void fold_summaries(int first, int last, int step, int m, int stride,
+__global__ __launch_bounds__(256) void fold_summaries(int bh0, int first, int last, int step, int m, int stride,
         const float *__restrict__ start, float *__restrict__ part)
 {
-    const int bh = blockIdx.x / (HEAD * HEAD / 256), el = (blockIdx.x % (HEAD * HEAD / 256)) * 256 + threadIdx.x;
+    const int bh = bh0 + blockIdx.x / (HEAD * HEAD / 256), el = (blockIdx.x % (HEAD * HEAD / 256)) * 256 + threadIdx.x;
     const int key = el / HEAD;
     float *pp = part + (size_t)bh * stride * PART;
     float S = start ? start[(size_t)bh * HEAD * HEAD + el] : 0.f;
@@ -1161,13 +1178,30 @@ static SegPlan plan_segments(int BH, int Tlen) {
     if (nseg * m > MAX_SEG) { m = std::max(1, MAX_SEG / nseg); pps = (sps + m - 1) / m; m = (sps + pps - 1) / pps; }
     return SegPlan{nseg, sps, m, pps};
 }
+// Two groups of (batch, head) pairs.  When B*H is more than a whole number of CU rounds, the whole rounds run their
+// sequences in one piece (group A: the first nA pairs, no summary pass at all) and only the remainder is cut in time
+// (group B), so that it fills one more, shorter round: 320 pairs = 256 whole + 64 x 4 segments instead of 320 x 4.
+struct GroupPlan { int nA; SegPlan a, b; };
+static GroupPlan plan_groups(int BH, int Tlen) {
+    const int nsb = (Tlen + SB - 1) / SB;
+    GroupPlan p{0, SegPlan{1, nsb, 1, nsb}, plan_segments(BH, Tlen)};
+    const int whole = BH / 256 * 256, rest = BH - whole;
+    if (forced_segments() > 0 || whole == 0 || rest == 0) return p;
+    const SegPlan r = plan_segments(rest, Tlen);
+    auto cost = [](int bh, const SegPlan &x) {
+        return (double)((bh * x.nseg + 255) / 256) * (x.sps + 1) * (x.nseg > 1 ? 1.3 : 1.0);
+    };
+    if (cost(whole, p.a) + cost(rest, r) < 0.97 * cost(BH, p.b)) { p.nA = whole; p.b = r; }
+    return p;
+}
 static size_t part_bytes(int B, int H) { return (size_t)B * H * MAX_SEG * PART * sizeof(float); }
 
 // workspace of a forward call: checkpoints | forward segment summaries
 size_t forward_workspace(int B, int Tlen, int H) { return checkpoint_bytes(B, Tlen, H) + part_bytes(B, H); }
-// workspace of a backward call: the forward's | backward segment summaries | gu, gw partials (B*MAX_SEG, C)
+// workspace of a backward call: the forward's | backward segment summaries | gu, gw partials, each (B, C) for the
+// unsplit group and (B*MAX_SEG, C) for the split one
 size_t backward_workspace(int B, int Tlen, int C, int H) {
-    return forward_workspace(B, Tlen, H) + part_bytes(B, H) + 2 * (size_t)B * MAX_SEG * C * sizeof(float);
+    return forward_workspace(B, Tlen, H) + part_bytes(B, H) + 2 * (size_t)B * (MAX_SEG + 1) * C * sizeof(float);
 }
 
 template <class K>
@@ -1186,34 +1220,41 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    const int nsb = (Tlen + SB - 1) / SB;
-    const SegPlan pl = workspace ? plan_segments(B * H, Tlen) : SegPlan{1, nsb, 1, nsb};
+    const int nsb = (Tlen + SB - 1) / SB, BH = B * H;
+    const GroupPlan gp = workspace ? plan_groups(BH, Tlen) : GroupPlan{0, SegPlan{1, nsb, 1, nsb}, SegPlan{1, nsb, 1, nsb}};
     float *ckpt = (workspace && keep_ckpt) ? (float *)workspace : nullptr;
     float *part = workspace ? (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H)) : nullptr;
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v;
-    dim3 block(NT_F);
+    const SegPlan &pl = gp.b;
+    const int nB = BH - gp.nA;
     if (pl.nseg > 1) {
         const int pieces = (pl.nseg - 1) * pl.m;
-        dim3 grid(B * H * pieces);
+        dim3 grid(nB * pieces), block(NT_F);
         if (per_token)
-            hipLaunchKernelGGL((summary_pass<true, false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w,
-                               part, floor_decay);
+            hipLaunchKernelGGL((summary_pass<true, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk,
+                               vv, w, part, floor_decay);
         else
-            hipLaunchKernelGGL((summary_pass<false, false>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk, vv, w,
-                               part, floor_decay);
-        hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, 0, pieces - 1, 1, pl.m,
+            hipLaunchKernelGGL((summary_pass<false, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk,
+                               vv, w, part, floor_decay);
+        hipLaunchKernelGGL(fold_summaries, dim3(nB * (HEAD * HEAD / 256)), dim3(256), 0, s, gp.nA, 0, pieces - 1, 1, pl.m,
                            pl.nseg * pl.m, s_in, part);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(B * H * pl.nseg), block16(NT_F16);
-    prof_begin(KID_CHUNK_FORWARD, s);
-    if (per_token)
-        hipLaunchKernelGGL((forward16<true>), grid, block16, sizeof(Fwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
-                           vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
-    else
-        hipLaunchKernelGGL((forward16<false>), grid, block16, sizeof(Fwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
-                           vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+    dim3 block16(NT_F16);
+    auto launch = [&](int bh0, int n, const SegPlan &x) {
+        if (n <= 0) return;
+        dim3 grid(n * x.nseg);
+        if (per_token)
+            hipLaunchKernelGGL((forward16<true>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m, rr, kk,
+                               vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+        else
+            hipLaunchKernelGGL((forward16<false>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m, rr, kk,
+                               vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+    };
+    prof_begin(KID_CHUNK_FORWARD, s);          // (both groups count as the one forward kernel of the call)
+    launch(0, gp.nA, gp.a);
+    launch(gp.nA, nB, pl);
     prof_end(KID_CHUNK_FORWARD, s);
     return hipGetLastError();
 }
@@ -1224,8 +1265,8 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
                            void *workspace, bool have_ckpt, int floor_decay) {
     float *ckpt = (float *)workspace;
     float *gpart = (float *)((char *)workspace + forward_workspace(B, Tlen, H));
-    float *gu_part = (float *)((char *)gpart + part_bytes(B, H));
-    float *gw_part = gu_part + (size_t)B * MAX_SEG * C;
+    float *gu_one = (float *)((char *)gpart + part_bytes(B, H)), *gu_many = gu_one + (size_t)B * C;
+    float *gw_one = gu_many + (size_t)B * MAX_SEG * C, *gw_many = gw_one + (size_t)B * C;
     if (!have_ckpt) {      // the forward call did not leave its checkpoints here: rebuild them
         hipError_t e = forward_launch(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, workspace,
                                       true, floor_decay);
@@ -1238,37 +1279,47 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    const SegPlan pl = plan_segments(B * H, Tlen);
+    const int BH = B * H;
+    const GroupPlan gp = plan_groups(BH, Tlen);
+    const SegPlan &pl = gp.b;
+    const int nB = BH - gp.nA;
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v, *gg = (const bf16 *)gy;
     if (pl.nseg > 1) {
         const int pieces = (pl.nseg - 1) * pl.m;
-        dim3 grid(B * H * pieces), block(NT_F);
+        dim3 grid(nB * pieces), block(NT_F);
         if (per_token)
-            hipLaunchKernelGGL((summary_pass<true, true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, gg, w,
-                               gpart, floor_decay);
+            hipLaunchKernelGGL((summary_pass<true, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr,
+                               gg, w, gpart, floor_decay);
         else
-            hipLaunchKernelGGL((summary_pass<false, true>), grid, block, 0, s, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr, gg, w,
-                               gpart, floor_decay);
-        hipLaunchKernelGGL(fold_summaries, dim3(B * H * (HEAD * HEAD / 256)), dim3(256), 0, s, pl.nseg * pl.m - 1, pl.m,
+            hipLaunchKernelGGL((summary_pass<false, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr,
+                               gg, w, gpart, floor_decay);
+        hipLaunchKernelGGL(fold_summaries, dim3(nB * (HEAD * HEAD / 256)), dim3(256), 0, s, gp.nA, pl.nseg * pl.m - 1, pl.m,
                            -1, pl.m, pl.nseg * pl.m, gs_out, gpart);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(B * H * pl.nseg), block16(NT_B16);
-    prof_begin(KID_CHUNK_BACKWARD, s);
-    if (per_token)
-        hipLaunchKernelGGL((backward16<true>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
-                           vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part, gs_in,
-                           floor_decay);
-    else
-        hipLaunchKernelGGL((backward16<false>), grid, block16, sizeof(Bwd16Tiles), s, Tlen, C, H, pl.nseg, pl.sps, pl.m, rr, kk,
-                           vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr, gw_part,
-                           gu_part, gs_in, floor_decay);
+    dim3 block16(NT_B16);
+    auto launch = [&](int bh0, int n, const SegPlan &x, float *gw_part, float *gu_part) {
+        if (n <= 0) return;
+        dim3 grid(n * x.nseg);
+        if (per_token)
+            hipLaunchKernelGGL((backward16<true>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
+                               rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part,
+                               gs_in, floor_decay);
+        else
+            hipLaunchKernelGGL((backward16<false>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
+                               rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr,
+                               gw_part, gu_part, gs_in, floor_decay);
+    };
+    prof_begin(KID_CHUNK_BACKWARD, s);         // (both groups count as the one backward kernel of the call)
+    launch(0, gp.nA, gp.a, gw_one, gu_one);
+    launch(gp.nA, nB, pl, gw_many, gu_many);
     prof_end(KID_CHUNK_BACKWARD, s);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B * pl.nseg, C, gu_part, gu);
-    if (!per_token) hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B * pl.nseg, C, gw_part, gw);
+    hipLaunchKernelGGL(sum_partials, dim3((C + 255) / 256), dim3(256), 0, s, B, H, gp.nA, pl.nseg, gu_one, gu_many, gu);
+    if (!per_token)
+        hipLaunchKernelGGL(sum_partials, dim3((C + 255) / 256), dim3(256), 0, s, B, H, gp.nA, pl.nseg, gw_one, gw_many, gw);
     return hipGetLastError();
 }
 
