@@ -441,7 +441,24 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
         }
         scan_local(lc, ic, sm.wtot, w16, g, n);
     };
-    scan_ahead(rowA.w);
+    // Time-invariant decay (WKV5): in a step with all 64 tokens present the scaling factors depend only on the
+    // token's place p in its block, e^{excl} = w^p and e^{b-incl} = w^(15-p), and the block's decay is w^16: a lane
+    // keeps its eight factors for the whole kernel and needs no running sum and no exponential per step.
+    float Fr[4] = {1.f, 1.f, 1.f, 1.f}, Fk[4] = {1.f, 1.f, 1.f, 1.f};
+    if (!PER_TOKEN_W) {
+        const float lcst[4] = {l_const.x, l_const.y, l_const.z, l_const.w};
+        const int pl = tok & 15;
+#pragma unroll
+        for (int c = 0; c < 4; c++) { Fr[c] = exp2_fast(pl * lcst[c]); Fk[c] = exp2_fast((15 - pl) * lcst[c]); }
+        if (pl == 15) {
+            *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(exp2_fast(16.f * lcst[0]), exp2_fast(16.f * lcst[1]), exp2_fast(16.f * lcst[2]), exp2_fast(16.f * lcst[3]));
+            *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(exp2_fast(-16.f * lcst[0]), exp2_fast(-16.f * lcst[1]), exp2_fast(-16.f * lcst[2]), exp2_fast(-16.f * lcst[3]));
+        }
+    }
+    auto whole_step = [&](int sb) { return !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
+#pragma unroll
+    for (int c = 0; c < 4; c++) lc[c] = ic[c] = 0.f;
+    if (!whole_step(sb0)) scan_ahead(rowA.w);
     lds_barrier();
     PT_DECL
     // one step; `cur` holds its inputs (and takes those of the step after the next), `nxt` those of the next step
@@ -459,14 +476,21 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
                 const int t = (sb - 1) * SB + tok;
                 if (t < Tlen) *reinterpret_cast<uint2 *>(y + base + (size_t)t * C + c4) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
             }
-            scan_join(inc, tot, sm.wtot, w16, n);
+            const bool whole = whole_step(sb);
             float rhv[4], khv[4], p = 0.f;
+            if (whole) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                rhv[c] = rf[c] * exp2_fast(inc[c] - l[c]);
-                khv[c] = kf[c] * exp2_fast(tot[c] - inc[c]);
-                p = fmaf(rf[c] * uf[c], kf[c], p);
+                for (int c = 0; c < 4; c++) { rhv[c] = rf[c] * Fr[c]; khv[c] = kf[c] * Fk[c]; }
+            } else {
+                scan_join(inc, tot, sm.wtot, w16, n);
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    rhv[c] = rf[c] * exp2_fast(inc[c] - l[c]);
+                    khv[c] = kf[c] * exp2_fast(tot[c] - inc[c]);
+                }
             }
+#pragma unroll
+            for (int c = 0; c < 4; c++) p = fmaf(rf[c] * uf[c], kf[c], p);
             uint32_t h0, l0, h1, l1;
             const int o = tok * LD + c4, ot = tok * LDT + c4;
             split2(rhv[0], rhv[1], h0, l0); split2(rhv[2], rhv[3], h1, l1);
@@ -476,7 +500,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             *reinterpret_cast<uint2 *>(&sm.kh[ot]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.khl[ot]) = make_uint2(l0, l1);
             *reinterpret_cast<uint2 *>(&sm.v[ot]) = pv;
-            if ((w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
+            if (!whole && (w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
                 if (g == 3) {
                     *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(exp2_fast(tot[0]), exp2_fast(tot[1]), exp2_fast(tot[2]), exp2_fast(tot[3]));
                     *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(exp2_fast(-tot[0]), exp2_fast(-tot[1]), exp2_fast(-tot[2]), exp2_fast(-tot[3]));
@@ -563,7 +587,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
 #pragma unroll
             for (int e = 0; e < 4; e++) sm.rh[(16 * q + 4 * g + e) * LD + 16 * wv + n] = bf16_bits(yt[e]);
         }
-        if (sb + 1 < sb1) scan_ahead(nxt.w);
+        if (sb + 1 < sb1 && !whole_step(sb + 1)) scan_ahead(nxt.w);
         PT_MARK(4)
         lds_barrier();
         have_y = y != nullptr;
@@ -723,14 +747,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     const int c4 = 4 * n, tok = 4 * w16 + g;
 
     bool have_out = false;
-    float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (!PER_TOKEN_W) {
-        const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
-        l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
-                              log2_decay(w4.w, floor_decay));
-    }
     uint2 pr, pk, pv, pg;
-    float4 pw;
+    float4 pw = make_float4(0.f, 0.f, 0.f, 0.f);      // per-token decay only (the time-invariant one is read where it is used)
     auto fetch = [&](int sb, int tok, int c4) {       // (tok, c4 handed in: see WKV_LOCAL_LANE)
         const int t = sb * SB + tok;
         if (t < Tlen) {
@@ -739,10 +757,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             pk = *reinterpret_cast<const uint2 *>(k + o);
             pv = *reinterpret_cast<const uint2 *>(v + o);
             pg = *reinterpret_cast<const uint2 *>(gy + o);
-            pw = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+            if (PER_TOKEN_W) pw = *reinterpret_cast<const float4 *>(wraw + o);
         } else {
             pr = pk = pv = pg = make_uint2(0u, 0u);
-            pw = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (PER_TOKEN_W) pw = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
         }
     };
     const int lane0 = lane;
@@ -759,10 +777,34 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         }
     };
 
+    // Time-invariant decay (WKV5): in a step with all 64 tokens present the scaling factors depend only on the
+    // token's place p in its block, e^{excl} = w^p and e^{b-incl} = w^(15-p), and every block decays by w^16.  They
+    // are kept as two [16][64] tables in the (then unused) log w table; such a step needs no running sum, no
+    // exponential and one barrier less.  A step with missing tokens (the last of the sequence) takes the general way
+    // and overwrites the tables.
+    float *const tab_r = sm.lw, *const tab_k = sm.lw + 16 * HEAD;
+    bool tables_valid = false;
+    auto whole_step = [&](int sb) { return !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
+
     fetch(sb1 - 1, tok, c4);
     PT_DECL
     for (int sb = sb1 - 1; sb >= sb0; sb--) {
       PT_MARK(5)
+      const bool whole = whole_step(sb);
+      if (whole && !tables_valid) {
+          const int key = tid & 63, pl = tid >> 6;
+          const float lk = log2_decay(wraw[h * HEAD + key], floor_decay);
+          tab_r[pl * HEAD + key] = exp2_fast(pl * lk);
+          tab_k[pl * HEAD + key] = exp2_fast((15 - pl) * lk);
+          if (pl < 4) {
+              sm.tot[pl][key] = 16.f * lk;
+              sm.dec[pl][key] = exp2_fast(16.f * lk);
+              sm.ent[pl][key] = exp2_fast(-16.f * lk);
+          }
+          tables_valid = true;
+          lds_barrier();
+      }
+      if (!whole) tables_valid = false;
       {
         WKV_LOCAL_LANE
         // the step's checkpoint: loads issued now are back when the chains start
@@ -784,18 +826,31 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             if (PER_TOKEN_W) {
 #pragma unroll
                 for (int c = 0; c < 4; c++) l[c] = log2_decay(l[c], floor_decay);
+            } else if (!whole) {       // a step with missing tokens: they count as w = 1
+                const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+                const bool in = sb * SB + tok < Tlen;
+                l[0] = in ? log2_decay(w4.x, floor_decay) : 0.f; l[1] = in ? log2_decay(w4.y, floor_decay) : 0.f;
+                l[2] = in ? log2_decay(w4.z, floor_decay) : 0.f; l[3] = in ? log2_decay(w4.w, floor_decay) : 0.f;
             }
             if (have_out) write_out(sb + 1, tok, c4);
-            scan_local(l, inc, sm.wtot, w16, g, n);      // (the one-step-ahead form of forward16 costs registers this kernel lacks)
-            lds_barrier();
-            scan_join(inc, tot, sm.wtot, w16, n);
             float rhv[4], khv[4], p = 0.f;
+            if (whole) {
+                const float4 fr = *reinterpret_cast<const float4 *>(&tab_r[(tok & 15) * HEAD + c4]);
+                const float4 fk = *reinterpret_cast<const float4 *>(&tab_k[(tok & 15) * HEAD + c4]);
+                rhv[0] = rf[0] * fr.x; rhv[1] = rf[1] * fr.y; rhv[2] = rf[2] * fr.z; rhv[3] = rf[3] * fr.w;
+                khv[0] = kf[0] * fk.x; khv[1] = kf[1] * fk.y; khv[2] = kf[2] * fk.z; khv[3] = kf[3] * fk.w;
+            } else {
+                scan_local(l, inc, sm.wtot, w16, g, n);      // (the one-step-ahead form of forward16 costs registers this kernel lacks)
+                lds_barrier();
+                scan_join(inc, tot, sm.wtot, w16, n);
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                rhv[c] = rf[c] * exp2_fast(inc[c] - l[c]);
-                khv[c] = kf[c] * exp2_fast(tot[c] - inc[c]);
-                p = fmaf(rf[c] * uf[c], kf[c], p);
+                for (int c = 0; c < 4; c++) {
+                    rhv[c] = rf[c] * exp2_fast(inc[c] - l[c]);
+                    khv[c] = kf[c] * exp2_fast(tot[c] - inc[c]);
+                }
             }
+#pragma unroll
+            for (int c = 0; c < 4; c++) p = fmaf(rf[c] * uf[c], kf[c], p);
             uint32_t h0, l0, h1, l1;
             const int o = tok * LD + c4;
             *reinterpret_cast<uint2 *>(&sm.gy[o]) = pg;
@@ -809,9 +864,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             *reinterpret_cast<uint4 *>(&sm.rk[tok * HEAD + c4]) =
                 make_uint4((pr.x & 0xffffu) | (pk.x << 16), (pr.x >> 16) | (pk.x & 0xffff0000u),
                            (pr.y & 0xffffu) | (pk.y << 16), (pr.y >> 16) | (pk.y & 0xffff0000u));
-            *reinterpret_cast<float4 *>(&sm.incl[tok * HEAD + c4]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
-            *reinterpret_cast<float4 *>(&sm.lw[tok * HEAD + c4]) = make_float4(l[0], l[1], l[2], l[3]);
-            if ((w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
+            if (!whole) {
+                *reinterpret_cast<float4 *>(&sm.incl[tok * HEAD + c4]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
+                *reinterpret_cast<float4 *>(&sm.lw[tok * HEAD + c4]) = make_float4(l[0], l[1], l[2], l[3]);
+            }
+            if (!whole && (w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
                 if (g == 3) {
                     *reinterpret_cast<float4 *>(&sm.tot[q][c4]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
                     *reinterpret_cast<float4 *>(&sm.dec[q][c4]) = make_float4(exp2_fast(tot[0]), exp2_fast(tot[1]), exp2_fast(tot[2]), exp2_fast(tot[3]));
@@ -1003,8 +1060,16 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int tk = 16 * q + 4 * g + e;
-                const float inc = sm.incl[tk * HEAD + own], l = sm.lw[tk * HEAD + own], exc = inc - l;
-                const float E1 = exp2_fast(exc), E2 = exp2_fast(tot_i - inc);
+                float l = 0.f, E1, E2;
+                if (whole) {
+                    E1 = tab_r[(4 * g + e) * HEAD + own];
+                    E2 = tab_k[(4 * g + e) * HEAD + own];
+                } else {
+                    const float inc = sm.incl[tk * HEAD + own];
+                    l = sm.lw[tk * HEAD + own];
+                    E1 = exp2_fast(inc - l);
+                    E2 = exp2_fast(tot_i - inc);
+                }
                 const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
                 const uint32_t rkv = sm.rk[tk * HEAD + own];
                 const float rr = bf_lo(rkv), kr = bf_hi(rkv);
