@@ -661,7 +661,7 @@ struct Bwd16Tiles {
     uint16_t rhl[SB * LD];
     uint16_t kh[SB * LD];    // k e^{b-incl}    [token][key]
     uint16_t khl[SB * LD];
-    float incl[SB * HEAD];   // inclusive running log decay inside the block [token][key]
+    float incl[SB * HEAD];   // inclusive running log decay inside the block [token][key]; after the block phase the inside-block part of the decay gradient
     float lw[SB * HEAD];     // log w                                         [token][key]
     uint32_t rk[SB * HEAD];  // r and k as they came (bf16 pair: r low, k high)                 [token][key]
     float tot[4][HEAD];      // b per block and key
@@ -675,8 +675,8 @@ struct Bwd16Tiles {
     float pdiag[4][16];      // P[t][t]
     uint4 amat[4][64];       // A~ masked to t >= s (diagonal r.(u o k)), A-operand fragments (head, remainder)
     float tots[4][HEAD];     // per block and key: sum over the block's tokens of r gr - k gk
-    float arun[HEAD];        // the running sum at the end of the current step
-    float red[2][4][HEAD];   // gu / gw partial sums of the four block groups
+    float arun[2][HEAD];     // the running sum of the decay gradient at the end of a step (two copies, used in turn)
+    float red[4][HEAD];      // gu partial sums of the four block groups
     float4 kg3[4][64];       // kh G of the step's last block, parked here by wavefronts 8-11 (they are short of registers)
 };
 constexpr int NT_B16 = 1024;
@@ -738,10 +738,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                     for (int e = 0; e < 4; e++) a = fmaf(gp[own * HEAD + 16 * kk + 4 * g + e], cp[kk * 1024 + e * 4], a);
             }
             a = group_sum4(a);
-            if (g == 0) sm.arun[own] = a;
+            if (g == 0) sm.arun[0][own] = a;
         }
     }
-    float gu_acc = 0.f, gw_acc = 0.f;
+    float gu_acc = 0.f;
+    float4 gw_acc = make_float4(0.f, 0.f, 0.f, 0.f);      // time-invariant w: sum over this lane's tokens, channels c4..c4+3
 
     // preparing role: token tok of the step (block q), channels c4..c4+3 (one 128-byte row per 16 lanes)
     const int c4 = 4 * n, tok = 4 * w16 + g;
@@ -764,18 +765,46 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         }
     };
     const int lane0 = lane;
-    // gr, gk, gv (and gw) of a finished step wait in the rh, kh, v tiles (and the incl table), [token][channel];
-    // they leave as full rows, written by the lanes that overwrite those entries next
-    auto write_out = [&](int sb, int tok, int c4) {
+    // gr, gk, gv of a finished step wait in the rh, kh, v tiles, [token][channel]; they leave as full rows, written
+    // by the lanes that overwrite those entries next.  The decay gradient is finished on the way out:
+    //   dL/dlog w_t = (running sum at the end of the token's block) + (inside-block part, waiting in the incl table),
+    // the first being the sum at the step's end (arun[par]) plus the totals of the step's later blocks.
+    auto write_out = [&](int sb, int tok, int c4, int par) {
         const int t = sb * SB + tok;
+        float4 A = *reinterpret_cast<const float4 *>(&sm.arun[par][c4]);
+        const float4 t1 = *reinterpret_cast<const float4 *>(&sm.tots[1][c4]), t2 = *reinterpret_cast<const float4 *>(&sm.tots[2][c4]);
+        const float4 t3 = *reinterpret_cast<const float4 *>(&sm.tots[3][c4]);
+        if (w16 == 0) {             // wavefront-uniform
+            if (tok == 0) {         // the sum at the end of the step before (in time): into the other copy
+                const float4 t0 = *reinterpret_cast<const float4 *>(&sm.tots[0][c4]);
+                *reinterpret_cast<float4 *>(&sm.arun[par ^ 1][c4]) =
+                    make_float4(A.x + ((t0.x + t1.x) + (t2.x + t3.x)), A.y + ((t0.y + t1.y) + (t2.y + t3.y)),
+                                A.z + ((t0.z + t1.z) + (t2.z + t3.z)), A.w + ((t0.w + t1.w) + (t2.w + t3.w)));
+            }
+        }
+        if (q < 3) { A.x += t3.x; A.y += t3.y; A.z += t3.z; A.w += t3.w; }
+        if (q < 2) { A.x += t2.x; A.y += t2.y; A.z += t2.z; A.w += t2.w; }
+        if (q < 1) { A.x += t1.x; A.y += t1.y; A.z += t1.z; A.w += t1.w; }
+        const float4 D = *reinterpret_cast<const float4 *>(&sm.incl[tok * HEAD + c4]);
+        A.x += D.x; A.y += D.y; A.z += D.z; A.w += D.w;
         if (t < Tlen) {
             const size_t o = base + (size_t)t * C + c4;
             *reinterpret_cast<uint2 *>(gr + o) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
             *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
             *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
-            if (PER_TOKEN_W) *reinterpret_cast<float4 *>(gw_tok + o) = *reinterpret_cast<const float4 *>(&sm.incl[tok * HEAD + c4]);
+            if (PER_TOKEN_W) {      // dL/dw_raw = dL/dlog w x log w (natural logarithm); nothing where the floor holds
+                const float4 l4 = *reinterpret_cast<const float4 *>(&sm.lw[tok * HEAD + c4]);
+                const float lf[4] = {l4.x, l4.y, l4.z, l4.w};
+                float f[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) f[c] = (floor_decay && lf[c] <= LOG2_W_FLOOR) ? 0.f : lf[c] * LN2;
+                *reinterpret_cast<float4 *>(gw_tok + o) = make_float4(A.x * f[0], A.y * f[1], A.z * f[2], A.w * f[3]);
+            } else {
+                gw_acc.x += A.x; gw_acc.y += A.y; gw_acc.z += A.z; gw_acc.w += A.w;
+            }
         }
     };
+    int par = 0;
 
     // Time-invariant decay (WKV5): in a step with all 64 tokens present the scaling factors depend only on the
     // token's place p in its block, e^{excl} = w^p and e^{b-incl} = w^(15-p), and every block decays by w^16.  They
@@ -832,7 +861,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                 l[0] = in ? log2_decay(w4.x, floor_decay) : 0.f; l[1] = in ? log2_decay(w4.y, floor_decay) : 0.f;
                 l[2] = in ? log2_decay(w4.z, floor_decay) : 0.f; l[3] = in ? log2_decay(w4.w, floor_decay) : 0.f;
             }
-            if (have_out) write_out(sb + 1, tok, c4);
+            if (have_out) { write_out(sb + 1, tok, c4, par); par ^= 1; }
             float rhv[4], khv[4], p = 0.f;
             if (whole) {
                 const float4 fr = *reinterpret_cast<const float4 *>(&tab_r[(tok & 15) * HEAD + c4]);
@@ -1028,7 +1057,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         lds_barrier();
         PT_MARK(3)
 
-        float Dloc[4], lfac[4];
       {
         WKV_LOCAL_LANE
         if (role == 2) {
@@ -1060,14 +1088,13 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int tk = 16 * q + 4 * g + e;
-                float l = 0.f, E1, E2;
+                float E1, E2;
                 if (whole) {
                     E1 = tab_r[(4 * g + e) * HEAD + own];
                     E2 = tab_k[(4 * g + e) * HEAD + own];
                 } else {
                     const float inc = sm.incl[tk * HEAD + own];
-                    l = sm.lw[tk * HEAD + own];
-                    E1 = exp2_fast(inc - l);
+                    E1 = exp2_fast(inc - sm.lw[tk * HEAD + own]);
                     E2 = exp2_fast(tot_i - inc);
                 }
                 const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
@@ -1078,7 +1105,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                 const float gkv = gkn + u_i * rr * pd;
                 c[e] = rr * grv - kr * gkv;
                 z[e] = kr * gkn;
-                lfac[e] = (floor_decay && l <= LOG2_W_FLOOR) ? 0.f : l * LN2;       // back to the natural logarithm
                 gu_acc = fmaf(rr * kr, pd, gu_acc);
                 // this wavefront was the only reader left of its (block, quarter) corner of the rh and kh tiles
                 sm.rh[tk * LD + own] = bf16_bits(grv);
@@ -1089,36 +1115,19 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
             const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
             const float all = group_sum4(mine);
-            Dloc[0] = later + suf0 - z[0];
-            Dloc[1] = later + suf1 - z[1];
-            Dloc[2] = later + suf2 - z[2];
-            Dloc[3] = later - z[3];
+            // (the incl entries of this block and quarter had this wavefront as their only reader)
+            sm.incl[(16 * q + 4 * g + 0) * HEAD + own] = later + suf0 - z[0];
+            sm.incl[(16 * q + 4 * g + 1) * HEAD + own] = later + suf1 - z[1];
+            sm.incl[(16 * q + 4 * g + 2) * HEAD + own] = later + suf2 - z[2];
+            sm.incl[(16 * q + 4 * g + 3) * HEAD + own] = later - z[3];
             if (g == 0) sm.tots[q][own] = all;
         }
       }
         PT_MARK(4)
         lds_barrier();
-        {
-            WKV_LOCAL_LANE
-            float A_end = sm.arun[own];          // at the end of block q: the step's end plus the later blocks
-#pragma unroll
-            for (int qq = 3; qq >= 1; qq--) A_end += qq > q ? sm.tots[qq][own] : 0.f;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int t = sb * SB + 16 * q + 4 * g + e;
-                const float Dt = A_end + Dloc[e];
-                if (PER_TOKEN_W) {
-                    sm.incl[(16 * q + 4 * g + e) * HEAD + own] = Dt * lfac[e];
-                } else {
-                    gw_acc += (t < Tlen) ? Dt : 0.f;
-                }
-            }
-        }
-        lds_barrier();
-        if (role == 0 && g == 0) sm.arun[own] += (sm.tots[0][own] + sm.tots[1][own]) + (sm.tots[2][own] + sm.tots[3][own]);
         have_out = true;
     }
-    if (have_out) write_out(sb0, tok, c4);
+    if (have_out) write_out(sb0, tok, c4, par);
 
     PT_PRINT("bwd16")
     if (role == 1 && gs_in && seg == 0) {
@@ -1128,19 +1137,24 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(G[kk][0], G[kk][1], G[kk][2], G[kk][3]);
     }
     gu_acc = group_sum4(gu_acc);
-    gw_acc = group_sum4(gw_acc);
-    if (g == 0) {
-        sm.red[0][q][own] = gu_acc;
-        sm.red[1][q][own] = gw_acc;
+    if (g == 0) sm.red[q][own] = gu_acc;
+    float *gw16 = sm.q1;            // [16][HEAD]; the q1 table is dead by now
+    if (!PER_TOKEN_W) {
+        gw_acc.x = group_sum4(gw_acc.x); gw_acc.y = group_sum4(gw_acc.y);
+        gw_acc.z = group_sum4(gw_acc.z); gw_acc.w = group_sum4(gw_acc.w);
+        if (g == 0) *reinterpret_cast<float4 *>(&gw16[w16 * HEAD + c4]) = gw_acc;
     }
     lds_barrier();
     if (q == 0 && g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
         const size_t po = ((size_t)(b * nseg + seg) * H + h) * HEAD + own;
-        gu_part[po] = (sm.red[0][0][own] + sm.red[0][1][own]) + (sm.red[0][2][own] + sm.red[0][3][own]);
+        gu_part[po] = (sm.red[0][own] + sm.red[1][own]) + (sm.red[2][own] + sm.red[3][own]);
         if (!PER_TOKEN_W) {
             bool fl;
             const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
-            gw_part[po] = fl ? 0.f : ((sm.red[1][0][own] + sm.red[1][1][own]) + (sm.red[1][2][own] + sm.red[1][3][own])) * l;
+            float sum = 0.f;
+#pragma unroll
+            for (int x = 0; x < 16; x++) sum += gw16[x * HEAD + own];
+            gw_part[po] = fl ? 0.f : sum * l;
         }
     }
 }
