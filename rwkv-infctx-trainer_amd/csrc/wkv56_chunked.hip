@@ -123,23 +123,6 @@ __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane g
     return x;
 }
 
-// collects N tokens of a channel pair (one packed pair per token) into two rows of a [channel][token] tile
-template <int N>
-struct Gather {
-    uint32_t a[N / 2], b[N / 2];
-    __device__ __forceinline__ void add(int x, uint32_t pair) {
-        if (x & 1) { a[x >> 1] |= pair << 16;   b[x >> 1] |= pair & 0xffff0000u; }
-        else       { a[x >> 1] = pair & 0xffffu; b[x >> 1] = pair >> 16; }
-    }
-    __device__ __forceinline__ void put(uint16_t *tile, int ot) const {
-#pragma unroll
-        for (int i = 0; i < N / 4; i++) {
-            *reinterpret_cast<uint2 *>(&tile[ot + 4 * i]) = make_uint2(a[2 * i], a[2 * i + 1]);
-            *reinterpret_cast<uint2 *>(&tile[ot + LD + 4 * i]) = make_uint2(b[2 * i], b[2 * i + 1]);
-        }
-    }
-};
-
 // One segment's summary for the time-parallel split: what the segment does to a
 // state handed in, S_out = decay o S_in + delta (forward), or to a state gradient
 // handed back (backward).  [key][value] fp32 plus one decay per key.
@@ -149,9 +132,10 @@ constexpr int PART = HEAD * HEAD + HEAD;
 // The main forward pass with the work of a 64-token step spread over 16 wavefronts
 // (four per SIMD).  A step runs in three phases separated by workgroup barriers:
 //
-//   prepare   all wavefronts: lane = (token of a block, four channels); a block's running
-//             log decay is a prefix sum over the 16 lanes of a DPP row.  Every tile is
-//             [token][channel]; the operands that the MFMAs want with the tokens along the
+//   prepare   all wavefronts: lane = (one token, four channels), 16 lanes = that token's
+//             128-byte row; a block's running log decay is summed inside the wavefront (four
+//             tokens) and joined across the block's four wavefronts through LDS.  Every tile
+//             is [token][channel]; the operands that the MFMAs want with the tokens along the
 //             contraction (k e^{b-incl}, v) come out of the transposing LDS read of gfx950.
 //   chains    wavefronts 0-7 own the state for good: wavefront (w, half) holds keys
 //             32*half..32*half+31 x values 16w..16w+15 in registers, walks it over the four
@@ -160,14 +144,13 @@ constexpr int PART = HEAD * HEAD + HEAD;
 //   finish    wavefront (q, w): y of block q, value columns 16w..16w+15 = the two shares
 //             + (intra-block matrix) v, converted and stored.
 constexpr int NT_F16 = 1024;
-constexpr int LDT = LD;       // tiles read through the transposing load use the same padded row length
 
 struct Fwd16Tiles {
     uint16_t rh[SB * LD];     // r e^{excl}       [token][key]  bf16 head / remainder
     uint16_t rhl[SB * LD];
-    uint16_t kh[SB * LDT];    // k e^{b-incl}     [token][key]   (read both ways)
-    uint16_t khl[SB * LDT];
-    uint16_t v[SB * LDT];     // v                [token][value] (read transposed)
+    uint16_t kh[SB * LD];    // k e^{b-incl}     [token][key]   (read both ways)
+    uint16_t khl[SB * LD];
+    uint16_t v[SB * LD];     // v                [token][value] (read transposed)
     float dec[4][HEAD];       // e^{b} per block and key
     float ent[4][HEAD];       // e^{-b}
     float rho[SB];            // r . (u o k) per token
@@ -424,7 +407,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             x.w = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
-    const int tro = tr_lane_offset(lane, LDT);
+    const int tro = tr_lane_offset(lane, LD);
     // the slot of this wavefront's two state tiles in a checkpoint (accumulator layout)
     const size_t ck_off = (size_t)bh * (nsb + 1) * HEAD * HEAD;
 
@@ -492,7 +475,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
 #pragma unroll
             for (int c = 0; c < 4; c++) p = fmaf(rf[c] * uf[c], kf[c], p);
             uint32_t h0, l0, h1, l1;
-            const int o = tok * LD + c4, ot = tok * LDT + c4;
+            const int o = tok * LD + c4, ot = tok * LD + c4;
             split2(rhv[0], rhv[1], h0, l0); split2(rhv[2], rhv[3], h1, l1);
             *reinterpret_cast<uint2 *>(&sm.rh[o]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.rhl[o]) = make_uint2(l0, l1);
@@ -533,13 +516,13 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
                 y1 = mma2(r0, r1, s0l, s1l, y1);
                 y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
                 // S <- e^{b} o S + (k e^{b-incl})^T v
-                const s4 v_op = frag_tr(sm.v, tro + (16 * blk) * LDT + 16 * wv);
+                const s4 v_op = frag_tr(sm.v, tro + (16 * blk) * LD + 16 * wv);
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][32 * hk + 16 * j + 4 * g]);
                     S[j][0] *= d4.x; S[j][1] *= d4.y; S[j][2] *= d4.z; S[j][3] *= d4.w;
-                    S[j] = mma2(frag_tr(sm.kh, tro + (16 * blk) * LDT + 32 * hk + 16 * j),
-                                frag_tr(sm.khl, tro + (16 * blk) * LDT + 32 * hk + 16 * j), v_op, v_op, S[j]);
+                    S[j] = mma2(frag_tr(sm.kh, tro + (16 * blk) * LD + 32 * hk + 16 * j),
+                                frag_tr(sm.khl, tro + (16 * blk) * LD + 32 * hk + 16 * j), v_op, v_op, S[j]);
                 }
                 y0 += y1 + y2;
                 sm.yi[hk][blk][wv][lane] = make_float4(y0[0], y0[1], y0[2], y0[3]);
@@ -580,7 +563,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
         if (y) {
             const float4 ya = sm.yi[0][q][wv][lane], yb = sm.yi[1][q][wv][lane];
             const uint4 am = sm.amat[q][lane];
-            const s4 v_op = frag_tr(sm.v, tro + (16 * q) * LDT + 16 * wv);
+            const s4 v_op = frag_tr(sm.v, tro + (16 * q) * LD + 16 * wv);
             f4 yt = {ya.x + yb.x, ya.y + yb.y, ya.z + yb.z, ya.w + yb.w};
             yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
             // into the rh tile (nobody reads it any more in this step), [token][value]; it leaves as full rows
