@@ -1212,6 +1212,9 @@ inline int &forced_piece_steps() {       // 0 = choose automatically
     static int v = [] { const char *e = getenv("RWKV_WKV_PPS"); return e ? atoi(e) : 0; }();
     return v;
 }
+// what the summary pass and the fold add to a run in n segments, as a factor on the main kernels' time
+// (the pass reads (n-1)/n of the tokens at about 40 % of the main kernels' cost per token)
+static double segment_overhead(int n) { return 1.0 + 0.4 * (n - 1) / n; }
 static SegPlan plan_segments(int BH, int Tlen) {
     const int nsb = (Tlen + SB - 1) / SB;
     const int forced = forced_segments();
@@ -1220,10 +1223,10 @@ static SegPlan plan_segments(int BH, int Tlen) {
         want = std::min(forced, nsb);
     } else {
         double best = 1e30;
-        for (int cand = 1; cand <= 16 && cand * 4 <= std::max(4, nsb); cand *= 2) {
+        for (int cand = 1; cand <= 16 && cand * 4 <= std::max(4, nsb); cand++) {
             const int sps = (nsb + cand - 1) / cand;
             const double rounds = (double)((BH * cand + 255) / 256);
-            const double cost = rounds * (sps + 1) * (cand > 1 ? 1.3 : 1.0);
+            const double cost = rounds * (sps + 1) * segment_overhead(cand);
             if (cost < best * 0.97) { best = cost; want = cand; }
         }
     }
@@ -1251,7 +1254,7 @@ static GroupPlan plan_groups(int BH, int Tlen) {
     if (forced_segments() > 0 || whole == 0 || rest == 0) return p;
     const SegPlan r = plan_segments(rest, Tlen);
     auto cost = [](int bh, const SegPlan &x) {
-        return (double)((bh * x.nseg + 255) / 256) * (x.sps + 1) * (x.nseg > 1 ? 1.3 : 1.0);
+        return (double)((bh * x.nseg + 255) / 256) * (x.sps + 1) * segment_overhead(x.nseg);
     };
     if (cost(whole, p.a) + cost(rest, r) < 0.97 * cost(BH, p.b)) { p.nA = whole; p.b = r; }
     return p;

@@ -352,7 +352,7 @@ def test_chunked_backward_rebuilds_checkpoints_when_not_given():
 
 
 @pytest.mark.parametrize("version", [5, 6])
-@pytest.mark.parametrize("nseg,T", [(1, 1024), (2, 1024), (4, 1024), (3, 1000), (8, 832)])
+@pytest.mark.parametrize("nseg,T", [(1, 1024), (2, 1024), (4, 1024), (3, 1000), (5, 1344), (8, 832)])
 def test_chunked_time_segments(version, nseg, T):
     """The time-parallel split (segment summaries folded in order) gives the same
     outputs and gradients as the oracle for any number of segments, ragged ones included."""
