@@ -43,6 +43,9 @@ def parse():
     ap.add_argument("--rotate", type=int, default=3, help="distinct input sets cycled through")
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"],
                     help="timed steps replayed from a HIP graph of one rotation period, or launched one by one")
+    ap.add_argument("--w-dtype", default="fp32", choices=["fp32", "bf16"],
+                    help="WKV6 only: dtype of the raw decay tensor and its gradient (fp32 is what the workload is "
+                         "defined with; bf16 is what a mixed-precision TimeMix hands over)")
     ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run three plain 256 MiB device copies first (reference point for the FETCH_SIZE / "
@@ -53,7 +56,7 @@ def parse():
 class Runner56:
     """WKV5 / WKV6 forward+backward through the C ABI on preallocated buffers."""
 
-    def __init__(self, cfg, algo, rotate):
+    def __init__(self, cfg, algo, rotate, w_dtype="fp32"):
         import torch
         from rwkv_wkv_hip import _lib, configs
         self.torch, self._lib, self.L = torch, _lib, _lib.lib()
@@ -64,6 +67,10 @@ class Runner56:
             self.sets.append({n: t.to(dev).contiguous() for n, t in wl.tensors.items()})
         self.wl = wl
         self.version = wl.version
+        self.w16 = w_dtype == "bf16" and wl.version == 6
+        if self.w16:
+            for st in self.sets:
+                st["w"] = st["w"].to(torch.bfloat16)
         B, T, C, H = wl.B, wl.T, wl.C, wl.H
         self.dims = (B, T, C, H)
         self.dt = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[wl.dtype]
@@ -86,13 +93,16 @@ class Runner56:
         self.tokens_per_step = B * T
         elems = B * T * C
         st = B * H * 64 * 64 * 4
-        per = 34 if self.version == 6 else 22
-        self.bytes_step = per * elems + 5 * st
-        self.bytes_fwd = (12 if self.version == 6 else 8) * elems + 2 * st
-        self.bytes_bwd = (22 if self.version == 6 else 14) * elems + 3 * st
+        wb = 2 if self.w16 else 4                       # bytes of a decay / decay-gradient element
+        fwd_b = (6 + wb + 2) if self.version == 6 else 8
+        bwd_b = (8 + wb + 6 + wb) if self.version == 6 else 14
+        self.bytes_step = (fwd_b + bwd_b) * elems + 5 * st
+        self.bytes_fwd = fwd_b * elems + 2 * st
+        self.bytes_bwd = bwd_b * elems + 3 * st
         self.dtype_name = "bf16"
-        self.desc = (f"cfg{cfg}: WKV{self.version} fwd+bwd B{B} T{T} C{C} H{H} head 64, bf16 r/k/v/dy, fp32 "
-                     f"raw decay and state, state carried step to step, state gradient fed back")
+        self.desc = (f"cfg{cfg}: WKV{self.version} fwd+bwd B{B} T{T} C{C} H{H} head 64, bf16 r/k/v/dy, "
+                     f"{'bf16' if self.w16 else 'fp32'} raw decay, fp32 state, state carried step to step, state "
+                     f"gradient fed back")
 
     def step(self):
         B, T, C, H = self.dims
@@ -100,7 +110,7 @@ class Runner56:
         s_in, s_out = self.state[self.i % 2], self.state[(self.i + 1) % 2]
         self.i += 1
         p = lambda t: t.data_ptr()
-        flags = self._lib.FLOOR_DECAY
+        flags = self._lib.FLOOR_DECAY | (self._lib.W_BF16 if self.w16 else 0)
         st = self.fwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
                       p(s["u"]), p(s_in), p(self.y), p(s_out), p(self.ws), self.ws.numel())
         assert st == 0, self.L.wkv_strerror(st)
@@ -274,7 +284,7 @@ def main():
         sys.exit(2)
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    runner = (Runner4 if a.cfg == 2 else Runner56)(a.cfg, a.algo, a.rotate)
+    runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype)
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
     if a.traffic_probe:
@@ -318,7 +328,7 @@ def main():
     achieved = dom_bytes / (kern[dom]["ms"] * 1e-3) / 1e9
     kname = f"{dom} (kernel id {kern[dom]['kernel_id']})"
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(a.cfg, a.algo, a.segments, kname),
+                "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(a.cfg, a.algo, a.segments, kname) if a.w_dtype == "fp32" else None,
                 "kernel": kname,
                 "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_ms": kern[dom]["ms"],
                 "kernels_ms": {k: v["ms"] for k, v in kern.items()},

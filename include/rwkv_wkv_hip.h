@@ -8,8 +8,8 @@
  *
  * Layouts (all contiguous, row-major):
  *   r, k, v, y, gy, gr, gk, gv   (B, T, C) in `dtype`          C = H * 64
- *   w (WKV6), gw (WKV6)          (B, T, C) fp32, RAW decay parameter:
- *                                the decay applied is exp(-exp(w))
+ *   w (WKV6), gw (WKV6)          (B, T, C) fp32 (bf16 with WKV_W_BF16), RAW decay
+ *                                parameter: the decay applied is exp(-exp(w))
  *   w (WKV5), gw (WKV5), u, gu   (H, 64)   fp32 (gw, gu summed over batch and time)
  *   state                        (B, H, 64, 64) fp32, [key index][value index]
  *   WKV4: time_decay, time_first (C) fp32;  state (B, C, 3) fp32 = (aa, bb, pp)
@@ -47,6 +47,12 @@ typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
 #define WKV_CHECKPOINTS_VALID 2u   /* backward only: the workspace passed is the one the matching
                                       forward call (same arguments, same algo) was given, so the
                                       state checkpoints it left there are used instead of rebuilt */
+
+#define WKV_W_BF16 4u         /* WKV6 with the chunked algorithm only: w and gw are bf16 (B, T, C), as a
+                                 mixed-precision TimeMix produces the decay and as the reference allocates its
+                                 gradient (RWKV-v6/src/module/TimeMix.py:50,90); w is widened to fp32 inside, as
+                                 the reference's w.float() does.  WKV_ERR_ALGO where the call would run token by
+                                 token */
 
 /* algorithm selector */
 #define WKV_ALGO_AUTO      0  /* chunked where it applies, else recurrent */
@@ -93,7 +99,7 @@ int wkv_profile_end(float *ms, int capacity);
  * WKV_CHECKPOINTS_VALID saves backward one sweep over k, v, w. */
 size_t wkv6_forward_workspace(int B, int T, int C, int H, int dtype, int algo);
 int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
-                 const void *r, const void *k, const void *v, const float *w, const float *u,
+                 const void *r, const void *k, const void *v, const void *w, const float *u,
                  const float *state_in, void *y, float *state_out,
                  void *workspace, size_t workspace_bytes);
 
@@ -101,9 +107,9 @@ size_t wkv6_backward_workspace(int B, int T, int C, int H, int dtype, int algo);
 /* gstate_out may be NULL (no gradient arrives through the state handed out,
  * i.e. truncated BPTT); gstate_in may be NULL when it is not wanted. */
 int wkv6_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
-                  const void *r, const void *k, const void *v, const float *w, const float *u,
+                  const void *r, const void *k, const void *v, const void *w, const float *u,
                   const float *state_in, const void *gy, const float *gstate_out,
-                  void *gr, void *gk, void *gv, float *gw, float *gu, float *gstate_in,
+                  void *gr, void *gk, void *gv, void *gw, float *gu, float *gstate_in,
                   void *workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------- WKV5 ----

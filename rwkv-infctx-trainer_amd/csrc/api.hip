@@ -34,7 +34,7 @@ int pick_algo56(int algo, int T, int dtype, unsigned flags) {
 }
 
 int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
-              const void *r, const void *k, const void *v, const float *w, const float *u, const float *state_in,
+              const void *r, const void *k, const void *v, const void *w, const float *u, const float *state_in,
               void *y, float *state_out, void *workspace, size_t workspace_bytes) {
     int st = check_dims56(B, T, C, H, dtype);
     if (st) return st;
@@ -44,17 +44,19 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
         if (!aligned16(p)) return WKV_ERR_ALIGN;
     const int a = pick_algo56(algo, T, dtype, flags);
     if (a < 0) return a;
+    const bool w16 = (flags & WKV_W_BF16) != 0;
+    if (w16 && (!per_token || a != WKV_ALGO_CHUNKED)) return WKV_ERR_ALGO;
     if (a == WKV_ALGO_CHUNKED) {
         // with a workspace the state at the start of every 64-token step is left there for backward
         if (workspace) {
             if (!aligned16(workspace)) return WKV_ERR_ALIGN;
             if (workspace_bytes < chunked::forward_workspace(B, T, H)) return WKV_ERR_WORKSPACE;
         }
-        hipError_t e = chunked::forward_launch((hipStream_t)stream, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
+        hipError_t e = chunked::forward_launch((hipStream_t)stream, per_token, w16, B, T, C, H, r, k, v, w, u, state_in, y,
                                                state_out, workspace, true, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
         return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
     }
-    hipError_t e = recurrent_forward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, y,
+    hipError_t e = recurrent_forward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, (const float *)w, u, state_in, y,
                                      state_out, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
@@ -74,8 +76,8 @@ size_t backward56_workspace(int B, int T, int C, int H, int dtype, int algo) {
 }
 
 int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
-               const void *r, const void *k, const void *v, const float *w, const float *u, const float *state_in,
-               const void *gy, const float *gstate_out, void *gr, void *gk, void *gv, float *gw, float *gu,
+               const void *r, const void *k, const void *v, const void *w, const float *u, const float *state_in,
+               const void *gy, const float *gstate_out, void *gr, void *gk, void *gv, void *gw, float *gu,
                float *gstate_in, void *workspace, size_t workspace_bytes) {
     int st = check_dims56(B, T, C, H, dtype);
     if (st) return st;
@@ -86,18 +88,20 @@ int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dty
         if (!aligned16(p)) return WKV_ERR_ALIGN;
     const int a = pick_algo56(algo, T, dtype, flags);
     if (a < 0) return a;
+    const bool w16 = (flags & WKV_W_BF16) != 0;
+    if (w16 && (!per_token || a != WKV_ALGO_CHUNKED)) return WKV_ERR_ALGO;
     if (!workspace) return WKV_ERR_NULL;
     if (workspace_bytes < (a == WKV_ALGO_CHUNKED ? chunked::backward_workspace(B, T, C, H)
                                                  : recurrent_backward_workspace(B, T, C)))
         return WKV_ERR_WORKSPACE;
     if (a == WKV_ALGO_CHUNKED) {
-        hipError_t e = chunked::backward_launch((hipStream_t)stream, per_token, B, T, C, H, r, k, v, w, u, state_in, gy,
+        hipError_t e = chunked::backward_launch((hipStream_t)stream, per_token, w16, B, T, C, H, r, k, v, w, u, state_in, gy,
                                                 gstate_out, gr, gk, gv, gw, gu, gstate_in, workspace,
                                                 (flags & WKV_CHECKPOINTS_VALID) != 0, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
         return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
     }
-    hipError_t e = recurrent_backward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, w, u, state_in, gy,
-                                      gstate_out, gr, gk, gv, gw, gu, gstate_in, (float *)workspace,
+    hipError_t e = recurrent_backward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, (const float *)w, u, state_in, gy,
+                                      gstate_out, gr, gk, gv, (float *)gw, gu, gstate_in, (float *)workspace,
                                       (flags & WKV_FLOOR_DECAY) ? 1 : 0);
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
@@ -175,7 +179,7 @@ size_t wkv5_forward_workspace(int B, int T, int C, int H, int dtype, int algo) {
 }
 
 int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
-                 const void *k, const void *v, const float *w, const float *u, const float *state_in, void *y,
+                 const void *k, const void *v, const void *w, const float *u, const float *state_in, void *y,
                  float *state_out, void *workspace, size_t workspace_bytes) {
     return forward56(true, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, y, state_out, workspace,
                      workspace_bytes);
@@ -195,8 +199,8 @@ size_t wkv5_backward_workspace(int B, int T, int C, int H, int dtype, int algo) 
 }
 
 int wkv6_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo, const void *r,
-                  const void *k, const void *v, const float *w, const float *u, const float *state_in, const void *gy,
-                  const float *gstate_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gstate_in,
+                  const void *k, const void *v, const void *w, const float *u, const float *state_in, const void *gy,
+                  const float *gstate_out, void *gr, void *gk, void *gv, void *gw, float *gu, float *gstate_in,
                   void *workspace, size_t workspace_bytes) {
     return backward56(true, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, gy, gstate_out, gr, gk, gv,
                       gw, gu, gstate_in, workspace, workspace_bytes);

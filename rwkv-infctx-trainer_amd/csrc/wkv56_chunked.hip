@@ -123,6 +123,28 @@ __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane g
     return x;
 }
 
+// The raw decay of one token's four channels as it waits in registers between fetch and use: fp32, or bf16 as a
+// mixed-precision TimeMix hands it over (W16; converted where it is used, so the prefetch holds half the registers
+// and moves half the bytes).  For the time-invariant decay the same slot carries the constant log decay.
+template <bool W16> struct WReg;
+template <> struct WReg<false> {
+    float4 v;
+    static __device__ __forceinline__ WReg load(const void *w, size_t o) {
+        return WReg{*reinterpret_cast<const float4 *>(static_cast<const float *>(w) + o)};
+    }
+    static __device__ __forceinline__ WReg from(float4 x) { return WReg{x}; }
+    __device__ __forceinline__ float4 f4() const { return v; }
+};
+template <> struct WReg<true> {
+    uint2 v;
+    static __device__ __forceinline__ WReg load(const void *w, size_t o) {
+        return WReg{*reinterpret_cast<const uint2 *>(static_cast<const bf16 *>(w) + o)};
+    }
+    static __device__ __forceinline__ WReg from(float4 x) { return WReg{make_uint2(bf16_pack2(x.x, x.y), bf16_pack2(x.z, x.w))}; }
+    __device__ __forceinline__ float4 f4() const { return make_float4(bf_lo(v.x), bf_hi(v.x), bf_lo(v.y), bf_hi(v.y)); }
+};
+#define WKV_NEG_INF4 make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY)
+
 // One segment's summary for the time-parallel split: what the segment does to a
 // state handed in, S_out = decay o S_in + delta (forward), or to a state gradient
 // handed back (backward).  [key][value] fp32 plus one decay per key.
@@ -239,9 +261,9 @@ struct PassTiles {
     float tot[4][HEAD];       // b
 };
 
-template <bool PER_TOKEN_W, bool BACKWARD>
+template <bool PER_TOKEN_W, bool BACKWARD, bool W16>
 __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, int H, int nseg, int sps, int m, int pps,
-        const bf16 *__restrict__ a_in, const bf16 *__restrict__ b_in, const float *__restrict__ wraw,
+        const bf16 *__restrict__ a_in, const bf16 *__restrict__ b_in, const void *__restrict__ wraw,
         float *__restrict__ part, int floor_decay)
 {
     __shared__ __align__(16) PassTiles sm;
@@ -262,12 +284,12 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
     const int c4 = 4 * n, tok0 = 16 * wv + 4 * g;
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
-        const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+        const float4 w4 = *reinterpret_cast<const float4 *>(static_cast<const float *>(wraw) + h * HEAD + c4);
         l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
                               log2_decay(w4.w, floor_decay));
     }
     uint2 pa[4], pb[4];
-    float4 pw[4];
+    WReg<W16> pw[4];
     auto fetch = [&](int sb) {
 #pragma unroll
         for (int x = 0; x < 4; x++) {
@@ -276,10 +298,10 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
                 const size_t o = base + (size_t)t * C + c4;
                 pa[x] = *reinterpret_cast<const uint2 *>(a_in + o);
                 pb[x] = *reinterpret_cast<const uint2 *>(b_in + o);
-                pw[x] = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+                pw[x] = PER_TOKEN_W ? WReg<W16>::load(wraw, o) : WReg<W16>::from(l_const);
             } else {
                 pa[x] = pb[x] = make_uint2(0u, 0u);
-                pw[x] = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+                pw[x] = WReg<W16>::from(PER_TOKEN_W ? WKV_NEG_INF4 : make_float4(0.f, 0.f, 0.f, 0.f));
             }
         }
     };
@@ -291,7 +313,8 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
             float l[4][4], inc[4][4], run[4] = {0.f, 0.f, 0.f, 0.f}, tot[4];
 #pragma unroll
             for (int x = 0; x < 4; x++) {
-                const float lw4[4] = {pw[x].x, pw[x].y, pw[x].z, pw[x].w};
+                const float4 pf = pw[x].f4();
+                const float lw4[4] = {pf.x, pf.y, pf.z, pf.w};
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     l[x][c] = PER_TOKEN_W ? log2_decay(lw4[c], floor_decay) : lw4[c];
@@ -355,10 +378,10 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
     if (wv == 0) pp[HEAD * HEAD + lane] = exp2_fast(dsum);
 }
 
-template <bool PER_TOKEN_W>
+template <bool PER_TOKEN_W, bool W16>
 __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
-        const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
+        const void *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
         bf16 *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt, const float *__restrict__ part,
         int floor_decay)
 {
@@ -387,12 +410,12 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
 
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!PER_TOKEN_W) {
-        const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+        const float4 w4 = *reinterpret_cast<const float4 *>(static_cast<const float *>(wraw) + h * HEAD + c4);
         l_const = make_float4(log2_decay(w4.x, floor_decay), log2_decay(w4.y, floor_decay), log2_decay(w4.z, floor_decay),
                               log2_decay(w4.w, floor_decay));
     }
     // the inputs of this lane's token, fetched two steps ahead into two register sets used in turn
-    struct Row { uint2 r, k, v; float4 w; };
+    struct Row { uint2 r, k, v; WReg<W16> w; };
     Row rowA, rowB;
     auto fetch = [&](int sb, Row &x) __attribute__((always_inline)) {
         const int t = sb * SB + tok;
@@ -401,10 +424,10 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             x.r = *reinterpret_cast<const uint2 *>(r + o);
             x.k = *reinterpret_cast<const uint2 *>(k + o);
             x.v = *reinterpret_cast<const uint2 *>(v + o);
-            x.w = PER_TOKEN_W ? *reinterpret_cast<const float4 *>(wraw + o) : l_const;
+            x.w = PER_TOKEN_W ? WReg<W16>::load(wraw, o) : WReg<W16>::from(l_const);
         } else {
             x.r = x.k = x.v = make_uint2(0u, 0u);
-            x.w = PER_TOKEN_W ? make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4(0.f, 0.f, 0.f, 0.f);
+            x.w = WReg<W16>::from(PER_TOKEN_W ? WKV_NEG_INF4 : make_float4(0.f, 0.f, 0.f, 0.f));
         }
     };
     const int tro = tr_lane_offset(lane, LD);
@@ -416,7 +439,8 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     if (sb0 + 1 < sb1) fetch(sb0 + 1, rowB);
     // log w of this lane's token and its running sum inside the wavefront, always one step ahead (see scan_local)
     float lc[4], ic[4];
-    auto scan_ahead = [&](const float4 &pw) __attribute__((always_inline)) {
+    auto scan_ahead = [&](const WReg<W16> &pwr) __attribute__((always_inline)) {
+        const float4 pw = pwr.f4();
         lc[0] = pw.x; lc[1] = pw.y; lc[2] = pw.z; lc[3] = pw.w;
         if (PER_TOKEN_W) {
 #pragma unroll
@@ -673,12 +697,12 @@ constexpr int NT_B16 = 1024;
               tok = 4 * w16 + g, tro = tr_lane_offset(lane, LD);                                              \
     (void)tro; (void)c4; (void)tok; (void)own;
 
-template <bool PER_TOKEN_W>
+template <bool PER_TOKEN_W, bool W16>
 __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
-        const float *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
+        const void *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
         const float *__restrict__ gs_out, const float *__restrict__ ckpt, const float *__restrict__ gpart,
-        bf16 *__restrict__ gr, bf16 *__restrict__ gk, bf16 *__restrict__ gv, float *__restrict__ gw_tok,
+        bf16 *__restrict__ gr, bf16 *__restrict__ gk, bf16 *__restrict__ gv, void *__restrict__ gw_tok,
         float *__restrict__ gw_part, float *__restrict__ gu_part, float *__restrict__ gs_in, int floor_decay)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -732,7 +756,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 
     bool have_out = false;
     uint2 pr, pk, pv, pg;
-    float4 pw = make_float4(0.f, 0.f, 0.f, 0.f);      // per-token decay only (the time-invariant one is read where it is used)
+    WReg<W16> pw = WReg<W16>::from(make_float4(0.f, 0.f, 0.f, 0.f));      // per-token decay only (the time-invariant one is read where it is used)
     auto fetch = [&](int sb, int tok, int c4) {       // (tok, c4 handed in: see WKV_LOCAL_LANE)
         const int t = sb * SB + tok;
         if (t < Tlen) {
@@ -741,10 +765,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             pk = *reinterpret_cast<const uint2 *>(k + o);
             pv = *reinterpret_cast<const uint2 *>(v + o);
             pg = *reinterpret_cast<const uint2 *>(gy + o);
-            if (PER_TOKEN_W) pw = *reinterpret_cast<const float4 *>(wraw + o);
+            if (PER_TOKEN_W) pw = WReg<W16>::load(wraw, o);
         } else {
             pr = pk = pv = pg = make_uint2(0u, 0u);
-            if (PER_TOKEN_W) pw = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            if (PER_TOKEN_W) pw = WReg<W16>::from(WKV_NEG_INF4);
         }
     };
     const int lane0 = lane;
@@ -781,7 +805,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                 float f[4];
 #pragma unroll
                 for (int c = 0; c < 4; c++) f[c] = (floor_decay && lf[c] <= LOG2_W_FLOOR) ? 0.f : lf[c] * LN2;
-                *reinterpret_cast<float4 *>(gw_tok + o) = make_float4(A.x * f[0], A.y * f[1], A.z * f[2], A.w * f[3]);
+                const float gw4[4] = {A.x * f[0], A.y * f[1], A.z * f[2], A.w * f[3]};
+                if (W16) store4(static_cast<bf16 *>(gw_tok) + o, gw4);
+                else store4(static_cast<float *>(gw_tok) + o, gw4);
             } else {
                 gw_acc.x += A.x; gw_acc.y += A.y; gw_acc.z += A.z; gw_acc.w += A.w;
             }
@@ -805,7 +831,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
       const bool whole = whole_step(sb);
       if (whole && !tables_valid) {
           const int key = tid & 63, pl = tid >> 6;
-          const float lk = log2_decay(wraw[h * HEAD + key], floor_decay);
+          const float lk = log2_decay(static_cast<const float *>(wraw)[h * HEAD + key], floor_decay);
           tab_r[pl * HEAD + key] = exp2_fast(pl * lk);
           tab_k[pl * HEAD + key] = exp2_fast((15 - pl) * lk);
           if (pl < 4) {
@@ -830,7 +856,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         }
         // ---------------- prepare the operands of this lane's token
         {
-            float l[4] = {pw.x, pw.y, pw.z, pw.w}, inc[4], tot[4];
+            const float4 pf = pw.f4();
+            float l[4] = {pf.x, pf.y, pf.z, pf.w}, inc[4], tot[4];
             const float rf[4] = {bf_lo(pr.x), bf_hi(pr.x), bf_lo(pr.y), bf_hi(pr.y)};
             const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
             const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
@@ -839,7 +866,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
                 for (int c = 0; c < 4; c++) l[c] = log2_decay(l[c], floor_decay);
             } else if (!whole) {       // a step with missing tokens: they count as w = 1
-                const float4 w4 = *reinterpret_cast<const float4 *>(wraw + h * HEAD + c4);
+                const float4 w4 = *reinterpret_cast<const float4 *>(static_cast<const float *>(wraw) + h * HEAD + c4);
                 const bool in = sb * SB + tok < Tlen;
                 l[0] = in ? log2_decay(w4.x, floor_decay) : 0.f; l[1] = in ? log2_decay(w4.y, floor_decay) : 0.f;
                 l[2] = in ? log2_decay(w4.z, floor_decay) : 0.f; l[3] = in ? log2_decay(w4.w, floor_decay) : 0.f;
@@ -1133,7 +1160,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         gu_part[po] = (sm.red[0][own] + sm.red[1][own]) + (sm.red[2][own] + sm.red[3][own]);
         if (!PER_TOKEN_W) {
             bool fl;
-            const float l = log_decay(wraw[h * HEAD + own], floor_decay, &fl);
+            const float l = log_decay(static_cast<const float *>(wraw)[h * HEAD + own], floor_decay, &fl);
             float sum = 0.f;
 #pragma unroll
             for (int x = 0; x < 16; x++) sum += gw16[x * HEAD + own];
@@ -1275,16 +1302,19 @@ static hipError_t allow_lds(K kernel, size_t bytes) {
 }
 
 // workspace == nullptr: single segment, no checkpoints kept
-hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
-                          const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
+// w16: the per-token decay is bf16 (per_token only)
+hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tlen, int C, int H, const void *r, const void *k,
+                          const void *v, const void *w, const float *u, const float *s_in, void *y, float *s_out,
                           void *workspace, bool keep_ckpt, int floor_decay) {
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = allow_lds(forward16<true>, sizeof(Fwd16Tiles));
-        if (e == hipSuccess) e = allow_lds(forward16<false>, sizeof(Fwd16Tiles));
+        hipError_t e = allow_lds(forward16<true, false>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow_lds(forward16<true, true>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow_lds(forward16<false, false>, sizeof(Fwd16Tiles));
         if (e != hipSuccess) return e;
         attr_done = true;
     }
+    const int mode = per_token ? (w16 ? 2 : 1) : 0;
     const int nsb = (Tlen + SB - 1) / SB, BH = B * H;
     const GroupPlan gp = workspace ? plan_groups(BH, Tlen) : GroupPlan{0, SegPlan{1, nsb, 1, nsb}, SegPlan{1, nsb, 1, nsb}};
     float *ckpt = (workspace && keep_ckpt) ? (float *)workspace : nullptr;
@@ -1295,12 +1325,15 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
     if (pl.nseg > 1) {
         const int pieces = (pl.nseg - 1) * pl.m;
         dim3 grid(nB * pieces), block(NT_F);
-        if (per_token)
-            hipLaunchKernelGGL((summary_pass<true, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk,
-                               vv, w, part, floor_decay);
+        if (mode == 2)
+            hipLaunchKernelGGL((summary_pass<true, false, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, kk, vv, w, part, floor_decay);
+        else if (mode == 1)
+            hipLaunchKernelGGL((summary_pass<true, false, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, kk, vv, w, part, floor_decay);
         else
-            hipLaunchKernelGGL((summary_pass<false, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, kk,
-                               vv, w, part, floor_decay);
+            hipLaunchKernelGGL((summary_pass<false, false, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, kk, vv, w, part, floor_decay);
         hipLaunchKernelGGL(fold_summaries, dim3(nB * (HEAD * HEAD / 256)), dim3(256), 0, s, gp.nA, 0, pieces - 1, 1, pl.m,
                            pl.nseg * pl.m, s_in, part);
         hipError_t e = hipGetLastError();
@@ -1310,12 +1343,15 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
     auto launch = [&](int bh0, int n, const SegPlan &x) {
         if (n <= 0) return;
         dim3 grid(n * x.nseg);
-        if (per_token)
-            hipLaunchKernelGGL((forward16<true>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m, rr, kk,
-                               vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+        if (mode == 2)
+            hipLaunchKernelGGL((forward16<true, true>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
+                               rr, kk, vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+        else if (mode == 1)
+            hipLaunchKernelGGL((forward16<true, false>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
+                               rr, kk, vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
         else
-            hipLaunchKernelGGL((forward16<false>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m, rr, kk,
-                               vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+            hipLaunchKernelGGL((forward16<false, false>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
+                               rr, kk, vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
     };
     prof_begin(KID_CHUNK_FORWARD, s);          // (both groups count as the one forward kernel of the call)
     launch(0, gp.nA, gp.a);
@@ -1324,27 +1360,28 @@ hipError_t forward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C,
     return hipGetLastError();
 }
 
-hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
-                           const void *v, const float *w, const float *u, const float *s_in, const void *gy,
-                           const float *gs_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gs_in,
+hipError_t backward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tlen, int C, int H, const void *r, const void *k,
+                           const void *v, const void *w, const float *u, const float *s_in, const void *gy,
+                           const float *gs_out, void *gr, void *gk, void *gv, void *gw, float *gu, float *gs_in,
                            void *workspace, bool have_ckpt, int floor_decay) {
     float *ckpt = (float *)workspace;
     float *gpart = (float *)((char *)workspace + forward_workspace(B, Tlen, H));
     float *gu_one = (float *)((char *)gpart + part_bytes(B, H)), *gu_many = gu_one + (size_t)B * C;
     float *gw_one = gu_many + (size_t)B * MAX_SEG * C, *gw_many = gw_one + (size_t)B * C;
     if (!have_ckpt) {      // the forward call did not leave its checkpoints here: rebuild them
-        hipError_t e = forward_launch(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, workspace,
+        hipError_t e = forward_launch(s, per_token, w16, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, workspace,
                                       true, floor_decay);
         if (e != hipSuccess) return e;
     }
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = allow_lds(backward16<true>, sizeof(Bwd16Tiles));
-        if (e == hipSuccess) e = allow_lds(backward16<false>, sizeof(Bwd16Tiles));
+        hipError_t e = allow_lds(backward16<true, false>, sizeof(Bwd16Tiles));
+        if (e == hipSuccess) e = allow_lds(backward16<true, true>, sizeof(Bwd16Tiles));
+        if (e == hipSuccess) e = allow_lds(backward16<false, false>, sizeof(Bwd16Tiles));
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    const int BH = B * H;
+    const int BH = B * H, mode = per_token ? (w16 ? 2 : 1) : 0;
     const GroupPlan gp = plan_groups(BH, Tlen);
     const SegPlan &pl = gp.b;
     const int nB = BH - gp.nA;
@@ -1352,12 +1389,15 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
     if (pl.nseg > 1) {
         const int pieces = (pl.nseg - 1) * pl.m;
         dim3 grid(nB * pieces), block(NT_F);
-        if (per_token)
-            hipLaunchKernelGGL((summary_pass<true, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr,
-                               gg, w, gpart, floor_decay);
+        if (mode == 2)
+            hipLaunchKernelGGL((summary_pass<true, true, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, rr, gg, w, gpart, floor_decay);
+        else if (mode == 1)
+            hipLaunchKernelGGL((summary_pass<true, true, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, rr, gg, w, gpart, floor_decay);
         else
-            hipLaunchKernelGGL((summary_pass<false, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m, pl.pps, rr,
-                               gg, w, gpart, floor_decay);
+            hipLaunchKernelGGL((summary_pass<false, true, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
+                               pl.pps, rr, gg, w, gpart, floor_decay);
         hipLaunchKernelGGL(fold_summaries, dim3(nB * (HEAD * HEAD / 256)), dim3(256), 0, s, gp.nA, pl.nseg * pl.m - 1, pl.m,
                            -1, pl.m, pl.nseg * pl.m, gs_out, gpart);
         hipError_t e = hipGetLastError();
@@ -1367,13 +1407,17 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
     auto launch = [&](int bh0, int n, const SegPlan &x, float *gw_part, float *gu_part) {
         if (n <= 0) return;
         dim3 grid(n * x.nseg);
-        if (per_token)
-            hipLaunchKernelGGL((backward16<true>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
-                               rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part, gu_part,
-                               gs_in, floor_decay);
+        if (mode == 2)
+            hipLaunchKernelGGL((backward16<true, true>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps,
+                               x.m, rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part,
+                               gu_part, gs_in, floor_decay);
+        else if (mode == 1)
+            hipLaunchKernelGGL((backward16<true, false>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps,
+                               x.m, rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part,
+                               gu_part, gs_in, floor_decay);
         else
-            hipLaunchKernelGGL((backward16<false>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
-                               rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (float *)nullptr,
+            hipLaunchKernelGGL((backward16<false, false>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps,
+                               x.m, rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (void *)nullptr,
                                gw_part, gu_part, gs_in, floor_decay);
     };
     prof_begin(KID_CHUNK_BACKWARD, s);         // (both groups count as the one backward kernel of the call)
@@ -1384,7 +1428,8 @@ hipError_t backward_launch(hipStream_t s, bool per_token, int B, int Tlen, int C
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(sum_partials, dim3((C + 255) / 256), dim3(256), 0, s, B, H, gp.nA, pl.nseg, gu_one, gu_many, gu);
     if (!per_token)
-        hipLaunchKernelGGL(sum_partials, dim3((C + 255) / 256), dim3(256), 0, s, B, H, gp.nA, pl.nseg, gw_one, gw_many, gw);
+        hipLaunchKernelGGL(sum_partials, dim3((C + 255) / 256), dim3(256), 0, s, B, H, gp.nA, pl.nseg, gw_one, gw_many,
+                           (float *)gw);
     return hipGetLastError();
 }
 

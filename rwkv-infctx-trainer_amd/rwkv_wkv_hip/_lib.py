@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("RWKV_WKV_LIB", os.path.join(_HERE, "librwkv_wkv_hip.s
 WKV_F32, WKV_BF16, WKV_F16 = 0, 1, 2
 FLOOR_DECAY = 1
 CHECKPOINTS_VALID = 2
+W_BF16 = 4          # WKV6, chunked algorithm: w and gw are bf16
 ALGO_AUTO, ALGO_RECURRENT, ALGO_CHUNKED = 0, 1, 2
 TUNE_SEGMENTS = 1
 

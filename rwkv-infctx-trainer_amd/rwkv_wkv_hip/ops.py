@@ -64,16 +64,26 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
 
+def _blocked(version, B, T, C, H, dtype):
+    """True when a call with these arguments takes the blocked (matrix-core) algorithm."""
+    L = _lib.lib()
+    fq = L.wkv5_forward_workspace if version == 5 else L.wkv6_forward_workspace
+    return T > 1 and dtype in _DT and fq(B, T, C, H, _DT[dtype], _algo) > 0
+
+
 def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad):
     """Returns y, new_state and, when a backward call will follow, the
     workspace in which the forward kernel left its state checkpoints (sized
-    for that backward call) together with the algorithm that was in force."""
+    for that backward call) together with the algorithm that was in force.
+    `w32` is fp32, or (WKV6, blocked algorithm) bf16 as it came."""
     L = _lib.lib()
     dt = _check_rkv(B, T, C, H, r, k, v)
     _on_gpu(r, k, v, w32, u32, s32)
     y = torch.empty_like(r)
     new_state = torch.empty_like(s32)
     flags = _lib.FLOOR_DECAY if T > 1 else 0
+    if w32.dtype == torch.bfloat16:
+        flags |= _lib.W_BF16
     algo = _algo
     fn, fq, bq = (L.wkv5_forward, L.wkv5_forward_workspace, L.wkv5_backward_workspace) if version == 5 else \
                  (L.wkv6_forward, L.wkv6_forward_workspace, L.wkv6_backward_workspace)
@@ -93,6 +103,8 @@ def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate, ws, alg
     gu = torch.empty_like(u32)
     gs = torch.empty_like(s32)
     flags = _lib.FLOOR_DECAY if T > 1 else 0
+    if w32.dtype == torch.bfloat16:
+        flags |= _lib.W_BF16           # gw comes back in bf16 too (torch.empty_like above)
     fn, wsq = (L.wkv5_backward, L.wkv5_backward_workspace) if version == 5 else (L.wkv6_backward, L.wkv6_backward_workspace)
     if ws is not None:
         flags |= _lib.CHECKPOINTS_VALID
@@ -139,14 +151,17 @@ class WKV_5(torch.autograd.Function):
 
 class WKV_6(torch.autograd.Function):
     """WKV6: per-token decay.  r,k,v (B,T,C); w (B,T,C) raw (any float dtype,
-    used in fp32); u (H,64); s (B,H,64,64) [key][value]."""
+    used in fp32; a bf16 w is read as it is by the blocked algorithm and its
+    gradient comes back in bf16, as in the reference, RWKV-v6/src/module/
+    TimeMix.py:50,90); u (H,64); s (B,H,64,64) [key][value]."""
 
     @staticmethod
     def forward(ctx, B, T, C, H, r, k, v, w, u, s):
         assert s.is_contiguous() and w.is_contiguous() and u.is_contiguous()
         assert s.shape == (B, H, HEAD, HEAD) and H * HEAD == C and w.shape == (B, T, C)
         u32 = u.float().contiguous().view(H, HEAD)
-        w32 = w.float()
+        native_w = w.dtype == torch.bfloat16 and r.dtype == torch.bfloat16 and _blocked(6, B, T, C, H, r.dtype)
+        w32 = w if native_w else w.float()
         s32 = s.float()
         need_grad = any(t.requires_grad for t in (r, k, v, w, u, s))
         with torch.no_grad():

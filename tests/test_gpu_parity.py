@@ -369,6 +369,37 @@ def test_chunked_time_segments(version, nseg, T):
     compare(got, ref, 2e-2, f"segments v{version}/n{nseg}/T{T}")
 
 
+@pytest.mark.parametrize("nseg,T", [(1, 200), (3, 1000)])
+def test_chunked_v6_takes_bf16_decay(nseg, T):
+    """The raw decay handed over in bf16 (what a mixed-precision TimeMix produces and the reference widens with
+    w.float(), RWKV-v6/src/module/TimeMix.py:50) is read as it is by the blocked kernels, and its gradient comes
+    back in bf16 (as the reference allocates it, :90): same results as the oracle on the widened tensor."""
+    import ctypes
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    wl = configs.make(3, B=2, T=T, C=128, H=2, dtype=torch.bfloat16)
+    wl.tensors["w"] = wl.tensors["w"].to(torch.bfloat16)
+    print(f"case bf16 decay nseg={nseg} T={T}", flush=True)
+    assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg) == 0
+    try:
+        got = run_gpu56(6, wl, algo="chunked")
+    finally:
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, 0) == 0
+    assert got["gw"].dtype == torch.bfloat16
+    wide = configs.make(3, B=2, T=T, C=128, H=2, dtype=torch.bfloat16)
+    wide.tensors["w"] = wl.tensors["w"].float()
+    ref = run_oracle56(6, wide)
+    compare(got, ref, 2e-2, f"bf16 decay n{nseg}/T{T}")
+    # token by token there is no bf16 decay at the C boundary: the entry point says so
+    B, C, H = wl.B, wl.C, wl.H
+    g = {n: x.to(dev()).contiguous() for n, x in wl.tensors.items()}
+    y, s = torch.empty_like(g["r"]), torch.empty_like(g["state"])
+    p = lambda x: ctypes.c_void_p(x.data_ptr())
+    st = L.wkv6_forward(None, B, T, C, H, 1, _lib.FLOOR_DECAY | _lib.W_BF16, 1, p(g["r"]), p(g["k"]), p(g["v"]), p(g["w"]),
+                        p(g["u"]), p(g["state"]), p(y), p(s), None, 0)
+    assert st == -7
+
+
 def test_chunked_needs_the_decay_floor():
     """T = 1 follows the reference's single-step branch (no floor on the decay); the blocked
     path's range analysis relies on the floor, so it refuses and 'auto' takes the per-token path."""
