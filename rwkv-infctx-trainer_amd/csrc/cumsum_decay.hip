@@ -37,9 +37,50 @@ __global__ __launch_bounds__(256) void cumsum_decay_kernel(int Bw, int Tlen, int
     }
 }
 
+// The same for a chunk length known at compile time: the chunk's log decays stay in registers, so w is read once
+// (CH independent loads per lane in flight) instead of once for the chunk total and once more for the tables.
+template <int CH>
+__global__ __launch_bounds__(256) void cumsum_decay_chunk(int Bw, int Tlen, int C, int per_token,
+        const float *__restrict__ w, float *__restrict__ log_w, float *__restrict__ incl,
+        float *__restrict__ inter, float *__restrict__ intra, float *__restrict__ chunk_sum)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int n = blockIdx.y, b = blockIdx.z, nchunk = Tlen / CH;
+    const size_t row0 = ((size_t)b * Tlen + (size_t)n * CH) * C + c;
+    const float fixed = per_token ? 0.f : log_decay(w[c], true);
+    float l[CH];
+    if (per_token) {
+#pragma unroll
+        for (int t = 0; t < CH; t++) l[t] = w[row0 + (size_t)t * C];
+    }
+    float total = 0.f;
+#pragma unroll
+    for (int t = 0; t < CH; t++) {
+        l[t] = per_token ? log_decay(l[t], true) : fixed;
+        total += l[t];
+    }
+    if (chunk_sum) chunk_sum[((size_t)b * nchunk + n) * C + c] = total;
+    float run = 0.f;
+#pragma unroll
+    for (int t = 0; t < CH; t++) {
+        const size_t o = row0 + (size_t)t * C;
+        run += l[t];
+        if (log_w) log_w[o] = l[t];
+        if (incl) incl[o] = run;
+        if (inter) inter[o] = total - run;
+        if (intra) intra[o] = run - l[t];
+    }
+}
+
 hipError_t cumsum_decay_launch(hipStream_t s, int Bw, int Tlen, int C, int chunk, int per_token, const float *w,
                                float *log_w, float *incl, float *inter, float *intra, float *chunk_sum) {
     dim3 grid((C + 255) / 256, Tlen / chunk, Bw);
+    if (chunk == 128) {         // the reference's chunk_len (RWKV-v5/src/module/rwkv_inner.py:12)
+        hipLaunchKernelGGL(cumsum_decay_chunk<128>, grid, dim3(256), 0, s, Bw, Tlen, C, per_token, w, log_w, incl, inter, intra,
+                           chunk_sum);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(cumsum_decay_kernel, grid, dim3(256), 0, s, Bw, Tlen, C, chunk, per_token, w, log_w, incl, inter,
                        intra, chunk_sum);
     return hipGetLastError();
