@@ -77,6 +77,34 @@ def test_full_shape_v5_v6(cfg):
         assert_close(L[n].grad, fast[gn], 2e-2, f"chain {gn}")
 
 
+@pytest.mark.parametrize("version", [5, 6])
+def test_more_pairs_than_one_round_of_compute_units(version):
+    """B*H = 260: the blocked path runs the first 256 (batch, head) pairs in one piece and cuts the other four in
+    time (two launches per kernel, two regions of partial sums).  All outputs against the per-token kernel, and
+    the oracle on one head of each group for every batch row (so the batch-summed gu / v5 gw are covered)."""
+    from rwkv_wkv_hip import configs
+    B, H, T = 5, 52, 1024
+    C = H * 64
+    wl = configs.make(1 if version == 5 else 3, B=B, T=T, C=C, H=H, dtype=torch.bfloat16)
+    print(f"case two groups v{version} B{B} H{H} T{T}", flush=True)
+    cpu = wl.tensors
+    t = {n: x.to(DEV) for n, x in cpu.items()}
+    fast = gpu_fwd_bwd(version, t, B, T, C, H, "chunked")
+    slow = gpu_fwd_bwd(version, t, B, T, C, H, "recurrent")
+    for n in fast:
+        assert_close(fast[n], slow[n], 2e-2, f"two groups v{version} blocked vs per-token {n}")
+    heads = [1, H - 1]             # (b, 1) is below pair 256 for every b; (4, 51) is pair 259
+    hs = lambda x: head_slice(x, B, T, H, heads)
+    sub_w = cpu["w"][heads] if version == 5 else hs(cpu["w"])
+    ref = O.wkv_op_grads(version, B, T, 128, 2, hs(cpu["r"]).float(), hs(cpu["k"]).float(), hs(cpu["v"]).float(), sub_w,
+                         cpu["u"][heads], cpu["state"][:, heads], hs(cpu["dy"]).float(), cpu["dstate"][:, heads])
+    pick = {"y": hs, "gr": hs, "gk": hs, "gv": hs,
+            "gw": (lambda x: x[heads]) if version == 5 else hs,
+            "gu": lambda x: x[heads], "state": lambda x: x[:, heads], "gstate": lambda x: x[:, heads]}
+    for n in ref:
+        assert_close(pick[n](fast[n].cpu()), ref[n], 2e-2, f"two groups v{version} oracle heads {heads} {n}")
+
+
 def test_full_shape_v4():
     import rwkv_wkv_hip as W
     from rwkv_wkv_hip import configs
