@@ -34,8 +34,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=600)      # 0.2 s of GPU time at cfg4: short runs measure the launch
+    ap.add_argument("--warmup", type=int, default=30)      # and synchronisation latencies of the host more than the kernels
     ap.add_argument("--cfg", type=int, default=4, choices=[1, 2, 3, 4])
     ap.add_argument("--algo", default="auto", choices=["auto", "recurrent", "chunked"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
