@@ -172,12 +172,11 @@ class Runner4:
         return {"forward": (3,), "backward": (4,)}
 
 
-def capture_period(runner, period):
-    """One period of steps (input rotation x state ping-pong) recorded into a HIP graph.
+def capture_steps(runner, nsteps):
+    """`nsteps` consecutive steps (input rotation x state ping-pong) recorded into a HIP graph.
     The library allocates nothing and synchronises nothing in a call, so its launches
     record as they are.  Returns None when the capture fails."""
     torch = runner.torch
-    assert runner.i % period == 0
     eager_stream, i0 = runner.stream, runner.i
     try:
         g = torch.cuda.CUDAGraph()
@@ -186,7 +185,7 @@ def capture_period(runner, period):
         with torch.cuda.stream(side):
             with torch.cuda.graph(g, stream=side):
                 runner.stream = torch.cuda.current_stream().cuda_stream
-                for _ in range(period):
+                for _ in range(nsteps):
                     runner.step()
         torch.cuda.current_stream().wait_stream(side)
         return g
@@ -196,6 +195,11 @@ def capture_period(runner, period):
         return None
     finally:
         runner.stream = eager_stream
+
+
+def capture_period(runner, period):
+    assert runner.i % period == 0
+    return capture_steps(runner, period)
 
 
 def time_kernel(runner, kid, steps):
@@ -265,14 +269,28 @@ def cpu_baseline(cfg, heads):
     return out
 
 
+def kernel_source_hash():
+    """Fingerprint of the kernel sources the library is built from (the counters of a
+    profiler run describe exactly one version of the kernels)."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(ROOT, "rwkv-infctx-trainer_amd", "csrc", "*.h*"))):
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(cfg, algo, segments, kernel):
     """HBM bytes per launch of the dominant kernel from the committed rocprofv3 counter
-    summary of this same workload (profiles/), or None when there is none for it."""
+    summary of this same workload and this same version of the kernel sources
+    (profiles/), or None when there is none that matches."""
     path = os.path.join(ROOT, "profiles", f"wkv6_cfg{cfg}_traffic.json")
     if not os.path.exists(path):
         return None
     rec = json.load(open(path))
-    same = rec.get("algo") == algo and rec.get("segments") == (segments or "auto") and rec.get("kernel") == kernel
+    same = (rec.get("algo") == algo and rec.get("segments") == (segments or "auto") and rec.get("kernel") == kernel
+            and rec.get("source_hash") == kernel_source_hash())
     return rec["traffic_bytes_per_launch"] if same else None
 
 
@@ -297,22 +315,39 @@ def main():
     for _ in range(-(-max(a.warmup, 1) // period) * period if a.launch == "graph" else a.warmup):
         runner.step()
     torch.cuda.synchronize()
-    graph = capture_period(runner, period) if a.launch == "graph" else None
+    # The K timed steps as few graph launches as possible: a body of whole rotation periods (at most ~60 steps,
+    # replayed K // body times) and one more graph with what is left, so that a short run (the 20-step default of
+    # an automated harness) measures the GPU and not the host's launch latencies.
+    body = tail = None
+    body_steps = min(a.steps, 60) // period * period
+    if a.launch == "graph" and body_steps > 0:
+        body = capture_steps(runner, body_steps)
+        if body is not None and a.steps % body_steps:
+            tail = capture_steps(runner, a.steps % body_steps)
+            if tail is None:
+                body = None
+    graph = body
     if graph is not None:
         graph.replay()                 # untimed: the first replay uploads the graph
+        if tail is not None:
+            tail.replay()
         torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record()
     if graph is not None:
-        for _ in range(a.steps // period):
+        for _ in range(a.steps // body_steps):
             graph.replay()
-        for _ in range(a.steps % period):
-            runner.step()
+        if tail is not None:
+            tail.replay()
     else:
         for _ in range(a.steps):
             runner.step()
+    ev1.record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_step = dt / a.steps * 1e3
+    ms_step_gpu = ev0.elapsed_time(ev1) / a.steps       # the same region by HIP events on the launch stream
     tok_s = runner.tokens_per_step * a.steps / dt
 
     # per-kernel launch durations (HIP events around the kernel, on its stream)
@@ -341,7 +376,9 @@ def main():
            "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": runner.dtype_name, "data": "synthetic",
            "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto",
-                      "launch": f"hip graph of {period} steps per replay" if graph is not None else "eager"},
+                      "launch": (f"hip graph of {body_steps} steps per replay" + (f" + one of {a.steps % body_steps}" if tail is not None else ""))
+                                if graph is not None else "eager"},
+           "ms_per_step_gpu_events": ms_step_gpu,
            "roofline": roofline}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(a.cfg, a.cpu_heads)

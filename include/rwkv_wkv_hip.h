@@ -34,7 +34,9 @@ typedef enum {
     WKV_ERR_ALIGN = -4,       /* a pointer is not 16-byte aligned */
     WKV_ERR_WORKSPACE = -5,   /* workspace smaller than the matching *_workspace() query */
     WKV_ERR_LAUNCH = -6,      /* HIP reported an error at launch */
-    WKV_ERR_ALGO = -7         /* algorithm not available for this shape / dtype */
+    WKV_ERR_ALGO = -7,        /* algorithm not available for this shape / dtype */
+    WKV_ERR_ALIAS = -8        /* state_out overlaps state_in: with a sequence cut into time segments the last
+                                 segment would write the new state while the first still reads the old one */
 } wkv_status;
 
 typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
@@ -97,6 +99,7 @@ int wkv_profile_end(float *ms, int capacity);
  * checkpoints there.  Passing that same buffer, sized by
  * wkv6_backward_workspace() (>= the forward size), to backward together with
  * WKV_CHECKPOINTS_VALID saves backward one sweep over k, v, w. */
+/* state_out must not overlap state_in (WKV_ERR_ALIAS); the same holds for wkv5_forward. */
 size_t wkv6_forward_workspace(int B, int T, int C, int H, int dtype, int algo);
 int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
                  const void *r, const void *k, const void *v, const void *w, const float *u,

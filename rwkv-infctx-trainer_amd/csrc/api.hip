@@ -42,6 +42,11 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
     for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
                           (const void *)state_out})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
+    {
+        const uintptr_t a0 = reinterpret_cast<uintptr_t>(state_in), b0 = reinterpret_cast<uintptr_t>(state_out);
+        const size_t bytes = (size_t)B * H * HEAD * HEAD * sizeof(float);
+        if (a0 < b0 + bytes && b0 < a0 + bytes) return WKV_ERR_ALIAS;
+    }
     const int a = pick_algo56(algo, T, dtype, flags);
     if (a < 0) return a;
     const bool w16 = (flags & WKV_W_BF16) != 0;
@@ -127,6 +132,7 @@ const char *wkv_strerror(int status) {
         case WKV_ERR_WORKSPACE: return "workspace too small";
         case WKV_ERR_LAUNCH: return "HIP launch failed";
         case WKV_ERR_ALGO: return "algorithm not available for this shape/dtype";
+        case WKV_ERR_ALIAS: return "state_out overlaps state_in";
         default: return "unknown status";
     }
 }

@@ -1232,11 +1232,11 @@ size_t checkpoint_bytes(int B, int Tlen, int H) {
 constexpr int MAX_SEG = 64;
 struct SegPlan { int nseg, sps, m, pps; };     // segments, steps per segment, pieces per segment, steps per piece
 inline int &forced_segments() {          // 0 = choose automatically
-    static int v = [] { const char *e = getenv("RWKV_WKV_NSEG"); return e ? atoi(e) : 0; }();
+    static int v = [] { const char *e = getenv("RWKV_WKV_NSEG"); return e ? std::min(std::max(atoi(e), 0), MAX_SEG) : 0; }();
     return v;
 }
 inline int &forced_piece_steps() {       // 0 = choose automatically
-    static int v = [] { const char *e = getenv("RWKV_WKV_PPS"); return e ? atoi(e) : 0; }();
+    static int v = [] { const char *e = getenv("RWKV_WKV_PPS"); return e ? std::max(atoi(e), 0) : 0; }();
     return v;
 }
 // what the summary pass and the fold add to a run in n segments, as a factor on the main kernels' time

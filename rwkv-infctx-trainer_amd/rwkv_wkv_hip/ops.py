@@ -127,7 +127,7 @@ class WKV_5(torch.autograd.Function):
         assert state.shape == (B, H, HEAD, HEAD) and H * HEAD == C
         u32 = u.float().contiguous().view(H, HEAD)
         w32 = w.view(H, HEAD)
-        need_grad = any(t.requires_grad for t in (state, r, k, v, w, u))
+        need_grad = any(ctx.needs_input_grad)        # all False under torch.no_grad(): no checkpoints kept then
         with torch.no_grad():
             y, new_state, ws, algo = _forward56(5, B, T, C, H, r, k, v, w32, u32, state, need_grad)
         ctx.dims = (B, T, C, H)
@@ -163,7 +163,7 @@ class WKV_6(torch.autograd.Function):
         native_w = w.dtype == torch.bfloat16 and r.dtype == torch.bfloat16 and _blocked(6, B, T, C, H, r.dtype)
         w32 = w if native_w else w.float()
         s32 = s.float()
-        need_grad = any(t.requires_grad for t in (r, k, v, w, u, s))
+        need_grad = any(ctx.needs_input_grad)
         with torch.no_grad():
             y, new_state, ws, algo = _forward56(6, B, T, C, H, r, k, v, w32, u32, s32, need_grad)
         ctx.dims = (B, T, C, H)
@@ -187,8 +187,10 @@ class WKV_6(torch.autograd.Function):
 
 def RUN_WKV5_CUDA(B, T, C, H, state, r, k, v, w, u):
     """The reference's calling convention (RWKV-v5/src/module/TimeMix.py:145-154):
-    returns y and leaves the new state in ``state``."""
-    y, new_state = WKV_5.apply(B, T, C, H, state, r, k, v, w, u)
+    returns y and leaves the new state in ``state``.  The operator works on a copy
+    of the incoming state, as the reference saves ``state.clone()`` (:60): the
+    tensor kept for backward must not be the one overwritten here."""
+    y, new_state = WKV_5.apply(B, T, C, H, state.clone(), r, k, v, w, u)
     with torch.no_grad():
         state.copy_(new_state)
     return y
@@ -196,8 +198,9 @@ def RUN_WKV5_CUDA(B, T, C, H, state, r, k, v, w, u):
 
 def RUN_WKV6STATE_CUDA(B, T, C, H, r, k, v, w, u, s):
     """The reference's calling convention (RWKV-v6/src/module/TimeMix.py:111-118):
-    returns y and leaves the new state in ``s``."""
-    y, new_state = WKV_6.apply(B, T, C, H, r, k, v, w, u, s)
+    returns y and leaves the new state in ``s`` (the operator works on a copy of
+    the incoming state, as the reference saves ``s.clone()``, :51)."""
+    y, new_state = WKV_6.apply(B, T, C, H, r, k, v, w, u, s.clone())
     with torch.no_grad():
         s.copy_(new_state)
     return y
@@ -217,7 +220,7 @@ class _WKV4(torch.autograd.Function):
         k, v, st = k.contiguous(), v.contiguous(), wkv_state.float().contiguous()
         y = torch.empty_like(k)
         new_state = torch.empty_like(st)
-        need_grad = any(t.requires_grad for t in (time_decay, time_first, k, v, wkv_state))
+        need_grad = any(ctx.needs_input_grad)
         ckpt = _workspace(L.wkv4_checkpoint_bytes(B, T, C), k.device) if need_grad else None
         check(L.wkv4_forward(_stream(), B, T, C, _DT[k.dtype], _ptr(td), _ptr(tf), _ptr(k), _ptr(v), _ptr(st),
                              _ptr(y), _ptr(new_state), _ptr(ckpt)), "wkv4_forward")

@@ -37,7 +37,7 @@ def test_header_symbols_exported(L):
 def test_version_and_messages(L):
     assert L.wkv_abi_version() == 1
     assert L.wkv_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert L.wkv_strerror(code) not in (b"ok", b"unknown status")
 
 
@@ -55,6 +55,9 @@ def test_argument_checks_return_before_any_launch(L):
     # misaligned pointer
     odd = ctypes.c_void_p(24)
     assert L.wkv6_forward(null, 1, 8, 64, 1, 1, 0, 0, odd, one, one, one, one, one, one, one, null, 0) == -4
+    # state_out overlapping state_in
+    assert L.wkv6_forward(null, 1, 8, 64, 1, 1, 0, 0, one, one, one, one, one, ctypes.c_void_p(4096), one,
+                          ctypes.c_void_p(4096 + 64), null, 0) == -8
     # backward: workspace too small
     need = L.wkv6_backward_workspace(1, 8, 64, 1, 1, 0)
     assert need > 0

@@ -1,9 +1,8 @@
-"""Parity at the full benchmark shapes.  The CPU oracle would take too long on
-whole tensors, so each case combines (a) the oracle on a subset of heads /
-channels, which is exact for those because heads (v5/v6) and channels (v4) are
-independent recurrences, (b) the per-token fp32 kernel as a second, independent
-device implementation of the whole tensor, and (c) size-independent properties
-(segment chaining, linearity)."""
+"""Parity at the full benchmark shapes: (a) the CPU oracle over the WHOLE tensors
+(one batch row at a time for v5/v6, to bound host memory; heads and batch rows
+are independent recurrences), (b) the per-token fp32 kernel as a second,
+independent device implementation, and (c) size-independent properties (segment
+chaining)."""
 import pytest
 import torch
 
@@ -34,6 +33,39 @@ def head_slice(x, B, T, H, heads):
     return x.view(B, T, H, 64)[:, :, heads].reshape(B, T, len(heads) * 64).contiguous()
 
 
+def oracle_by_batch_row(version, cpu, B, T, C, H):
+    """wkv_op_grads over all heads, one batch row per call; per-row gu / WKV5 gw summed."""
+    rows = []
+    for b in range(B):
+        sl = slice(b, b + 1)
+        w = cpu["w"] if version == 5 else cpu["w"][sl]
+        rows.append(O.wkv_op_grads(version, 1, T, C, H, cpu["r"][sl].float(), cpu["k"][sl].float(), cpu["v"][sl].float(),
+                                   w, cpu["u"], cpu["state"][sl], cpu["dy"][sl].float(), cpu["dstate"][sl]))
+    out = {}
+    for n in rows[0]:
+        if n == "gu" or (n == "gw" and version == 5):
+            out[n] = torch.stack([r[n] for r in rows]).sum(0)
+        else:
+            out[n] = torch.cat([r[n] for r in rows], 0)
+    return out
+
+
+def test_cfg0_wkv5_forward_fp32():
+    """The reference's own CPU-runnable case: WKV5 forward, B1 T512 C768 H12, fp32, zero state
+    (plus the backward of the same call), against the oracle at rtol 1e-3."""
+    from rwkv_wkv_hip import configs
+    wl = configs.make(0)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    print(f"case cfg0: v5 B{B} T{T} C{C} H{H} fp32", flush=True)
+    cpu = wl.tensors
+    t = {n: x.to(DEV) for n, x in cpu.items()}
+    got = gpu_fwd_bwd(5, t, B, T, C, H, "auto")
+    ref = O.wkv_op_grads(5, B, T, C, H, cpu["r"], cpu["k"], cpu["v"], cpu["w"], cpu["u"], cpu["state"], cpu["dy"],
+                         cpu["dstate"])
+    for n in ref:
+        assert_close(got[n].cpu(), ref[n], 1e-3, f"cfg0 {n}")
+
+
 @pytest.mark.parametrize("cfg", [1, 3])
 def test_full_shape_v5_v6(cfg):
     from rwkv_wkv_hip import configs
@@ -46,17 +78,10 @@ def test_full_shape_v5_v6(cfg):
     slow = gpu_fwd_bwd(version, t, B, T, C, H, "recurrent")
     for n in fast:
         assert_close(fast[n], slow[n], 2e-2, f"cfg{cfg} blocked vs per-token {n}")
-    # (a) oracle on two heads (all batches, so that the batch-summed gu / v5 gw are covered)
-    heads = [1, H - 2]
-    hs = lambda x: head_slice(x, B, T, H, heads)
-    sub_w = cpu["w"][heads] if version == 5 else hs(cpu["w"])
-    ref = O.wkv_op_grads(version, B, T, 128, 2, hs(cpu["r"]).float(), hs(cpu["k"]).float(), hs(cpu["v"]).float(), sub_w,
-                         cpu["u"][heads], cpu["state"][:, heads], hs(cpu["dy"]).float(), cpu["dstate"][:, heads])
-    pick = {"y": hs, "gr": hs, "gk": hs, "gv": hs,
-            "gw": (lambda x: x[heads]) if version == 5 else hs,
-            "gu": lambda x: x[heads], "state": lambda x: x[:, heads], "gstate": lambda x: x[:, heads]}
+    # (a) the oracle over every head of every batch row; gu (and the WKV5 gw) are sums over the batch
+    ref = oracle_by_batch_row(version, cpu, B, T, C, H)
     for n in ref:
-        assert_close(pick[n](fast[n].cpu()), ref[n], 2e-2, f"cfg{cfg} oracle heads {heads} {n}")
+        assert_close(fast[n].cpu(), ref[n], 2e-2, f"cfg{cfg} oracle {n}")
     # (c) one call over T == two chained calls over T/2, state gradient handed back
     import rwkv_wkv_hip as W
     h = T // 2
@@ -117,19 +142,16 @@ def test_full_shape_v4():
     y, s = W.wkv_op(L["time_decay"], L["time_first"], L["k"], L["v"], L["state"])
     torch.autograd.backward([y, s], [t["dy"], t["dstate"]])
     torch.cuda.synchronize()
-    # oracle on channels 0..63 and the last 64 (channels are independent chains)
-    for c0 in (0, C - 64):
-        sl = slice(c0, c0 + 64)
-        yr, sr = O4.forward(cpu["time_decay"][sl], cpu["time_first"][sl], cpu["k"][..., sl], cpu["v"][..., sl], cpu["state"][:, sl])
-        ref = O4.backward(cpu["time_decay"][sl], cpu["time_first"][sl], cpu["k"][..., sl], cpu["v"][..., sl],
-                          cpu["state"][:, sl], cpu["dy"][..., sl], cpu["dstate"][:, sl])
-        assert_close(y[..., sl], yr, 1e-3, "v4 y")
-        und = lambda st: st[..., :2].float().cpu() * torch.exp(st[..., 2:3].float().cpu())
-        assert_close(und(s[:, sl]), und(sr), 1e-3, "v4 state")
-        assert_close(L["time_decay"].grad[sl], ref[0], 2e-3, "v4 g_time_decay")
-        assert_close(L["time_first"].grad[sl], ref[1], 2e-3, "v4 g_time_first")
-        assert_close(L["k"].grad[..., sl], ref[2], 1e-3, "v4 gk")
-        assert_close(L["v"].grad[..., sl], ref[3], 1e-3, "v4 gv")
+    # the C oracle over all channels (channels are independent chains)
+    yr, sr = O4.forward(cpu["time_decay"], cpu["time_first"], cpu["k"], cpu["v"], cpu["state"])
+    ref = O4.backward(cpu["time_decay"], cpu["time_first"], cpu["k"], cpu["v"], cpu["state"], cpu["dy"], cpu["dstate"])
+    assert_close(y, yr, 1e-3, "v4 y")
+    und = lambda st: st[..., :2].float().cpu() * torch.exp(st[..., 2:3].float().cpu())
+    assert_close(und(s), und(sr), 1e-3, "v4 state")
+    assert_close(L["time_decay"].grad, ref[0], 2e-3, "v4 g_time_decay")
+    assert_close(L["time_first"].grad, ref[1], 2e-3, "v4 g_time_first")
+    assert_close(L["k"].grad, ref[2], 1e-3, "v4 gk")
+    assert_close(L["v"].grad, ref[3], 1e-3, "v4 gv")
     # chaining: T == T/2 + T/2 through the carried state
     h = T // 2
     y1, s1 = W.wkv_op(t["time_decay"], t["time_first"], t["k"][:, :h].contiguous(), t["v"][:, :h].contiguous(), t["state"])
@@ -139,14 +161,14 @@ def test_full_shape_v4():
 
 def test_long_context_chain_7b_shape():
     """cfg4: 64 consecutive 4096-token segments at B1 C4096 H64, fp32 state carried
-    segment to segment on the GPU, forward + backward per segment.  Four heads are
+    segment to segment on the GPU, forward + backward per segment.  All 64 heads are
     followed on the CPU oracle with their own carried state: per-segment outputs and
     gradients within tolerance and no drift of the carried state."""
     import rwkv_wkv_hip as W
     from rwkv_wkv_hip import configs
     B, T, C, H, NSEG = 1, 4096, 4096, 64, 64
-    heads = [0, 21, 42, 63]
-    hs = lambda x: head_slice(x, B, T, H, heads)
+    heads = list(range(H))
+    hs = lambda x: x
     state = None
     ref_state = None
     worst = {}

@@ -87,3 +87,32 @@ def test_timemix_bf16_in_place_wrappers(version):
     rel = ((y.float().cpu() - y_ref).norm() / y_ref.norm()).item()
     assert rel < 3e-2, f"timemix bf16 v{version} y: relative error {rel}"
     assert_close(s, s_ref, 6e-2, f"timemix bf16 v{version} state")
+
+
+@pytest.mark.parametrize("version", [5, 6])
+def test_in_place_wrappers_train(version):
+    """Training through the reference's in-place convention: forward with RUN_*, which overwrites the state
+    buffer, then backward.  Gradients equal those of the functional operators on the same inputs."""
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=2, T=128, C=128, H=2, dtype=torch.bfloat16)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.cuda() for n, x in wl.tensors.items()}
+    names = ("r", "k", "v", "w", "u")
+
+    def leaves():
+        return {n: g[n].clone().requires_grad_(True) for n in names}
+    La, Lb = leaves(), leaves()
+    st = g["state"].clone()
+    if version == 5:
+        y = W.RUN_WKV5_CUDA(B, T, C, H, st, La["r"], La["k"], La["v"], La["w"], La["u"])
+        y2, s2 = W.WKV_5.apply(B, T, C, H, g["state"], Lb["r"], Lb["k"], Lb["v"], Lb["w"], Lb["u"])
+    else:
+        y = W.RUN_WKV6STATE_CUDA(B, T, C, H, La["r"], La["k"], La["v"], La["w"], La["u"], st)
+        y2, s2 = W.WKV_6.apply(B, T, C, H, Lb["r"], Lb["k"], Lb["v"], Lb["w"], Lb["u"], g["state"])
+    y.backward(g["dy"])
+    y2.backward(g["dy"])
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2) and torch.equal(st, s2), "in-place wrapper and functional operator disagree"
+    for n in names:
+        assert torch.equal(La[n].grad, Lb[n].grad), f"gradient of {n} differs"
