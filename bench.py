@@ -11,10 +11,12 @@ in HBM.  Prints ONE JSON line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--cfg 1|2|3|4] [--algo auto|recurrent|chunked]
                     [--launch graph|eager]
 
-The K timed steps are launched from a HIP graph that holds one period of the
-input rotation (six steps; what is left of K after whole replays runs as plain
-launches), or as plain launches throughout with ``--launch eager`` (and whenever
-the capture fails).
+The K timed steps are launched from HIP graphs (one graph of K steps up to
+K = 128; beyond that a 120-step body replayed K // 120 times plus one graph with
+the rest), or as plain launches with ``--launch eager`` (and whenever the capture
+fails).  They are timed twice: between two HIP events on the launch stream with
+the queue primed (``ms_per_step``, ``value``) and between two device
+synchronisations by the host clock (``ms_per_step_host``).
 """
 import argparse
 import ctypes
@@ -46,6 +48,9 @@ def parse():
     ap.add_argument("--w-dtype", default="fp32", choices=["fp32", "bf16"],
                     help="WKV6 only: dtype of the raw decay tensor and its gradient (fp32 is what the workload is "
                          "defined with; bf16 is what a mixed-precision TimeMix hands over)")
+    ap.add_argument("--w-shift", type=float, default=0.0,
+                    help="WKV6 only: added to the raw decay parameter (negative = slower decay; -5 makes every channel "
+                         "remember for thousands of tokens, the worst case of the time-parallel split's summary passes)")
     ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run three plain 256 MiB device copies first (reference point for the FETCH_SIZE / "
@@ -56,7 +61,7 @@ def parse():
 class Runner56:
     """WKV5 / WKV6 forward+backward through the C ABI on preallocated buffers."""
 
-    def __init__(self, cfg, algo, rotate, w_dtype="fp32"):
+    def __init__(self, cfg, algo, rotate, w_dtype="fp32", w_shift=0.0):
         import torch
         from rwkv_wkv_hip import _lib, configs
         self.torch, self._lib, self.L = torch, _lib, _lib.lib()
@@ -68,6 +73,9 @@ class Runner56:
         self.wl = wl
         self.version = wl.version
         self.w16 = w_dtype == "bf16" and wl.version == 6
+        if w_shift and wl.version == 6:
+            for st in self.sets:
+                st["w"] = st["w"] + w_shift
         if self.w16:
             for st in self.sets:
                 st["w"] = st["w"].to(torch.bfloat16)
@@ -102,7 +110,7 @@ class Runner56:
         self.dtype_name = "bf16"
         self.desc = (f"cfg{cfg}: WKV{self.version} fwd+bwd B{B} T{T} C{C} H{H} head 64, bf16 r/k/v/dy, "
                      f"{'bf16' if self.w16 else 'fp32'} raw decay, fp32 state, state carried step to step, state "
-                     f"gradient fed back")
+                     f"gradient fed back" + (f", raw decay shifted by {w_shift}" if w_shift else ""))
 
     def step(self):
         B, T, C, H = self.dims
@@ -302,7 +310,7 @@ def main():
         sys.exit(2)
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype)
+    runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift)
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
     if a.traffic_probe:
@@ -315,11 +323,12 @@ def main():
     for _ in range(-(-max(a.warmup, 1) // period) * period if a.launch == "graph" else a.warmup):
         runner.step()
     torch.cuda.synchronize()
-    # The K timed steps as few graph launches as possible: a body of whole rotation periods (at most ~60 steps,
-    # replayed K // body times) and one more graph with what is left, so that a short run (the 20-step default of
-    # an automated harness) measures the GPU and not the host's launch latencies.
+    # The K timed steps as few graph launches as possible: up to 128 steps are ONE graph; a longer run replays a
+    # body of 120 steps (whole rotation periods) K // 120 times, plus one more graph with what is left.  A graph
+    # launch costs the host (and the idle GPU) about 0.2 ms, so a short run (the 20-step default of an automated
+    # harness) would otherwise measure launch latencies rather than the kernels.
     body = tail = None
-    body_steps = min(a.steps, 60) // period * period
+    body_steps = a.steps if a.steps <= 128 else 120
     if a.launch == "graph" and body_steps > 0:
         body = capture_steps(runner, body_steps)
         if body is not None and a.steps % body_steps:
@@ -332,23 +341,36 @@ def main():
         if tail is not None:
             tail.replay()
         torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    def run_k_steps():
+        if graph is not None:
+            for _ in range(a.steps // body_steps):
+                graph.replay()
+            if tail is not None:
+                tail.replay()
+        else:
+            for _ in range(a.steps):
+                runner.step()
+
+    # (1) the K steps between two device synchronisations, by the host's clock.  This includes the latency of the
+    # first launch (about 0.2 - 0.6 ms for a graph: the GPU idles until the launch arrives), which is a property
+    # of the host, not of the kernels, and weighs 10 % and more on a 20-step run.
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
+    run_k_steps()
+    torch.cuda.synchronize()
+    ms_step_host = (time.perf_counter() - t0) / a.steps * 1e3
+    # (2) the same K steps once more, between two HIP events on the launch stream, with two untimed plain steps
+    # queued in front so that the GPU is still busy when the timed launches arrive: the events then bracket
+    # exactly the K steps' execution.  This is the figure reported as ms_per_step / value.
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(2):
+        runner.step()
     ev0.record()
-    if graph is not None:
-        for _ in range(a.steps // body_steps):
-            graph.replay()
-        if tail is not None:
-            tail.replay()
-    else:
-        for _ in range(a.steps):
-            runner.step()
+    run_k_steps()
     ev1.record()
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_step = dt / a.steps * 1e3
-    ms_step_gpu = ev0.elapsed_time(ev1) / a.steps       # the same region by HIP events on the launch stream
-    tok_s = runner.tokens_per_step * a.steps / dt
+    ms_step = ev0.elapsed_time(ev1) / a.steps
+    tok_s = runner.tokens_per_step / (ms_step * 1e-3)
 
     # per-kernel launch durations (HIP events around the kernel, on its stream)
     ksteps = min(a.steps, 20)
@@ -378,7 +400,10 @@ def main():
            "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto",
                       "launch": (f"hip graph of {body_steps} steps per replay" + (f" + one of {a.steps % body_steps}" if tail is not None else ""))
                                 if graph is not None else "eager"},
-           "ms_per_step_gpu_events": ms_step_gpu,
+           "ms_per_step_host": ms_step_host,
+           "timing": "ms_per_step and value: HIP events on the launch stream around exactly the K steps, the queue "
+                     "primed with two untimed steps; ms_per_step_host: the same K steps between two device "
+                     "synchronisations by the host clock (includes the latency of the first launch)",
            "roofline": roofline}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(a.cfg, a.cpu_heads)

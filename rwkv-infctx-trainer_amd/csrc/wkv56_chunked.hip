@@ -245,21 +245,33 @@ __device__ __forceinline__ void scan_join(float (&inc)[4], float (&tot)[4], cons
 // Time-parallel split.  One piece (`pps` steps) of a segment, from a zero state
 // (gradient): what the piece does to a state handed in, X_out = decay o X_in + delta.
 //   BACKWARD = false: state summary over pieces of the segments 0..nseg-2 (reads k, v, w):
-//                     X <- e^{b} o X + (k e^{b-incl})^T v      per 16-token block, first to last;
+//                     delta = sum over the piece's tokens s of (k_s e^{(decay from s to the piece's end)})^T v_s;
 //   BACKWARD = true:  state-gradient summary over pieces of the segments 1..nseg-1 (reads r, gy, w):
-//                     X <- e^{b} o X + (r e^{excl})^T gy       per 16-token block, last to first.
-// fold_summaries then chains the pieces.  Four wavefronts; wavefront w prepares block w of
+//                     delta = sum over t of (r_t e^{(decay from the piece's start to t)})^T gy_t.
+// The main kernels chain the pieces in their prologues (chain_state / chain_gradient).  Four wavefronts; wavefront w prepares block w of
 // a step (lane = four consecutive tokens x four channels, 16 lanes = one 128-byte row, the
 // running log decay inside the lane and two shuffles across) and owns value columns
 // 16w..16w+15 of X.  Tiles are [token][channel]; the MFMA operands come out of the
 // transposing LDS read.
+//
+// The steps of a piece are walked AWAY from the boundary the summary is for (the state pass from the piece's
+// last step to its first, the gradient pass from its first to its last): a step's contribution T (its four
+// blocks chained from zero) enters as  X += e^{R} o T  with R the log decay between the step and the boundary,
+// which only grows in size.  Once e^{R} is below 2^-56 for every key, what is left of the piece cannot change
+// X any more (fp32 keeps 24 bits) and the walk stops; the piece's decay is then reported as exactly 0, which
+// tells whoever chains the summaries that nothing beyond this piece matters.  With a decay that forgets within
+// a few hundred tokens every piece reads a few steps instead of all of its steps; with a decay close to 1
+// nothing stops early and the pass costs what a full pass costs.
 struct PassTiles {
     uint16_t a[SB * LD];      // forward: k e^{b-incl};  backward: r e^{excl}     [token][key]   bf16 head of the value
     uint16_t al[SB * LD];     //                                                                 bf16 remainder
     uint16_t b[SB * LD];      // forward: v;             backward: gy             [token][value]
     float dec[4][HEAD];       // e^{b} per block and key
     float tot[4][HEAD];       // b
+    float fac[2][HEAD];       // e^{R} per key for this step / the next one
+    int stop;
 };
+constexpr float PASS_CUT_LOG2 = -56.f;
 
 template <bool PER_TOKEN_W, bool BACKWARD, bool W16>
 __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, int H, int nseg, int sps, int m, int pps,
@@ -268,18 +280,19 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
 {
     __shared__ __align__(16) PassTiles sm;
     const int units = (nseg - 1) * m;       // workgroups per (batch, head)
-    const int bh = bh0 + blockIdx.x / units, piece = (BACKWARD ? m : 0) + blockIdx.x % units, seg = piece / m, b = bh / H, h = bh % H;
+    const int bh = bh0 + blockIdx.x / units, piece = (BACKWARD ? m : 0) + blockIdx.x % units, seg = piece / m, j = piece % m;
+    const int b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
-    const int sb0 = seg * sps + (piece % m) * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
+    const int sb0 = seg * sps + j * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
     const int nsteps = sb1 - sb0;
 
     // X[kk][e] = X[key 16kk+4g+e][value 16wv+n]
     f4 X[4];
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) X[kk] = f4{0.f, 0.f, 0.f, 0.f};
-    float dsum = 0.f;                       // wavefront 0, lane = key: log of the piece's decay
+    float R = 0.f;                          // wavefront 0, lane = key: log2 of the decay between the boundary and the next step
     // preparing role: tokens tok0..tok0+3 of the step (block wv), channels c4..c4+3
     const int c4 = 4 * n, tok0 = 16 * wv + 4 * g;
     float4 l_const = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -306,9 +319,14 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
         }
     };
     const int tro = tr_lane_offset(lane, LD);
-    if (nsteps > 0) fetch(BACKWARD ? sb1 - 1 : sb0);
+    // the state pass walks back in time, the gradient pass forward
+    auto step_at = [&](int it) { return BACKWARD ? sb0 + it : sb1 - 1 - it; };
+    if (nsteps > 0) fetch(step_at(0));
+    if (tid < HEAD) sm.fac[0][tid] = 1.f;
+    if (tid == 0) sm.stop = 0;
+    bool stopped = false;
     for (int it = 0; it < nsteps; it++) {
-        const int sb = BACKWARD ? sb1 - 1 - it : sb0 + it;
+        const int par = it & 1;
         {
             float l[4][4], inc[4][4], run[4] = {0.f, 0.f, 0.f, 0.f}, tot[4];
 #pragma unroll
@@ -354,28 +372,97 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
             }
         }
         lds_barrier();
-        if (it + 1 < nsteps) fetch(BACKWARD ? sb - 1 : sb + 1);          // next step's loads fly during the MFMA phase
-        if (wv == 0) dsum += (sm.tot[0][lane] + sm.tot[1][lane]) + (sm.tot[2][lane] + sm.tot[3][lane]);
+        if (it + 1 < nsteps) fetch(step_at(it + 1));          // next step's loads fly during the MFMA phase
+        if (wv == 0) {      // lane = key: the decay up to the next step, and whether anything later can still matter
+            R += (sm.tot[0][lane] + sm.tot[1][lane]) + (sm.tot[2][lane] + sm.tot[3][lane]);
+            sm.fac[par ^ 1][lane] = exp2_fast(R);
+            float mx = R;
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            if (lane == 0 && mx < PASS_CUT_LOG2) sm.stop = 1;
+        }
+        // the step's own contribution, its four blocks chained from zero (first to last going forward, last to first going back)
+        f4 Tt[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int blk = BACKWARD ? 3 - i : i;
             const s4 b_op = frag_tr(sm.b, tro + (16 * blk) * LD + 16 * wv);
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][16 * kk + 4 * g]);
-                X[kk][0] *= d4.x; X[kk][1] *= d4.y; X[kk][2] *= d4.z; X[kk][3] *= d4.w;
-                X[kk] = mma2(frag_tr(sm.a, tro + (16 * blk) * LD + 16 * kk), frag_tr(sm.al, tro + (16 * blk) * LD + 16 * kk),
-                             b_op, b_op, X[kk]);
+                if (i == 0) {
+                    Tt[kk] = f4{0.f, 0.f, 0.f, 0.f};
+                } else {
+                    const float4 d4 = *reinterpret_cast<const float4 *>(&sm.dec[blk][16 * kk + 4 * g]);
+                    Tt[kk][0] *= d4.x; Tt[kk][1] *= d4.y; Tt[kk][2] *= d4.z; Tt[kk][3] *= d4.w;
+                }
+                Tt[kk] = mma2(frag_tr(sm.a, tro + (16 * blk) * LD + 16 * kk), frag_tr(sm.al, tro + (16 * blk) * LD + 16 * kk),
+                              b_op, b_op, Tt[kk]);
             }
         }
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const float4 f = *reinterpret_cast<const float4 *>(&sm.fac[par][16 * kk + 4 * g]);
+            X[kk][0] = fmaf(f.x, Tt[kk][0], X[kk][0]); X[kk][1] = fmaf(f.y, Tt[kk][1], X[kk][1]);
+            X[kk][2] = fmaf(f.z, Tt[kk][2], X[kk][2]); X[kk][3] = fmaf(f.w, Tt[kk][3], X[kk][3]);
+        }
         lds_barrier();
+        if (sm.stop) { stopped = true; break; }
     }
     float *pp = part + ((size_t)bh * nseg * m + piece) * PART;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
 #pragma unroll
         for (int e = 0; e < 4; e++) pp[(16 * kk + 4 * g + e) * HEAD + 16 * wv + n] = X[kk][e];
-    if (wv == 0) pp[HEAD * HEAD + lane] = exp2_fast(dsum);
+    if (wv == 0) pp[HEAD * HEAD + lane] = stopped ? 0.f : exp2_fast(R);
+}
+
+// Chaining the piece summaries, done by the main kernels for the state elements a lane holds.  A lane's
+// elements are X[i] = X[key ki[i]][value vi[i]], i < N.
+//   chain_state:    the state at the start of segment `seg` = the summaries of the pieces before it applied in
+//                   order to the state handed in.  Walked from the nearest piece backwards,
+//                       S = D_p + d_p o (D_{p-1} + d_{p-1} o ( ... + d_0 o S_in)),
+//                   i.e. S = sum_q (prod_{q < q' <= p} d_q') o D_q, so that the walk ends as soon as the running product
+//                   of the decays is 0 for all of the lane's keys (a piece that forgot everything reports exactly 0).
+//   chain_gradient: the state gradient at the end of segment `seg`, from the pieces after it and the gradient handed in,
+//                   walked forward in the same way.
+// The summaries are read two pieces at a time, deltas and decays together, so that the common cases (the nearest piece
+// forgot everything; two pieces per segment) take one round trip to memory.  ONE_KEY: all N elements share the key ki[0].
+template <int N, bool ONE_KEY>
+__device__ __forceinline__ void chain_summaries(float (&X)[N], const int (&ki)[N], const int (&vi)[N], const float *__restrict__ pieces,
+                                                int first, int count, int dir, const float *__restrict__ ends) {
+    constexpr int NK = ONE_KEY ? 1 : N;
+    float run[NK];
+#pragma unroll
+    for (int i = 0; i < N; i++) X[i] = 0.f;
+#pragma unroll
+    for (int k = 0; k < NK; k++) run[k] = 1.f;
+    bool alive = true;
+    for (int x = 0; x < count && alive; x += 2) {
+        float d[2][N], dc[2][NK];
+#pragma unroll
+        for (int bb = 0; bb < 2; bb++) {
+            const float *q = pieces + (size_t)(first + dir * min(x + bb, count - 1)) * PART;
+#pragma unroll
+            for (int i = 0; i < N; i++) d[bb][i] = q[ki[i] * HEAD + vi[i]];
+#pragma unroll
+            for (int k = 0; k < NK; k++) dc[bb][k] = q[HEAD * HEAD + ki[k]];
+        }
+#pragma unroll
+        for (int bb = 0; bb < 2; bb++) {
+            if (x + bb < count && alive) {
+                bool any = false;
+#pragma unroll
+                for (int i = 0; i < N; i++) X[i] = fmaf(run[ONE_KEY ? 0 : i], d[bb][i], X[i]);
+#pragma unroll
+                for (int k = 0; k < NK; k++) { run[k] *= dc[bb][k]; any |= run[k] != 0.f; }
+                alive = any;
+            }
+        }
+    }
+    if (alive && ends) {
+#pragma unroll
+        for (int i = 0; i < N; i++) X[i] = fmaf(run[ONE_KEY ? 0 : i], ends[ki[i] * HEAD + vi[i]], X[i]);
+    }
 }
 
 template <bool PER_TOKEN_W, bool W16>
@@ -399,11 +486,22 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     // chain wavefronts: S[j][e] = S[key 32hk+16j+4g+e][value 16wv+n]
     f4 S[2] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
     if (chain) {
-        const float *sp = seg == 0 ? s_in + (size_t)bh * HEAD * HEAD : part + ((size_t)bh * nseg * m + seg * m - 1) * PART;
+        if (seg == 0) {
+            const float *sp = s_in + (size_t)bh * HEAD * HEAD;
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+            for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) S[j][e] = sp[(32 * hk + 16 * j + 4 * g + e) * HEAD + 16 * wv + n];
+                for (int e = 0; e < 4; e++) S[j][e] = sp[(32 * hk + 16 * j + 4 * g + e) * HEAD + 16 * wv + n];
+        } else {      // the summaries of the pieces before this segment, chained onto the state handed in
+            float X[8];
+            int ki[8], vi[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) { ki[i] = 32 * hk + 16 * (i >> 2) + 4 * g + (i & 3); vi[i] = 16 * wv + n; }
+            chain_summaries<8, false>(X, ki, vi, part + (size_t)bh * nseg * m * PART, seg * m - 1, seg * m, -1,
+                               s_in + (size_t)bh * HEAD * HEAD);
+#pragma unroll
+            for (int i = 0; i < 8; i++) S[i >> 2][i & 3] = X[i];
+        }
     }
     // preparing role: token tok of the step (block q), channels c4..c4+3
     const int c4 = 4 * n, tok = 4 * w16 + g;
@@ -723,26 +821,44 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     //   wavefronts 8-11:  its gradient, G[kk][e] = G[key 16kk+4g+e][value own]
     f4 G[4] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
     {
-        // the last segment starts from gs_out, an earlier one from what fold_summaries left
-        const float *gp = seg == nseg - 1 ? (gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr)
-                                          : gpart + ((size_t)bh * nseg * m + (seg + 1) * m) * PART;
-        if (gp && (role == 1 || role == 2)) {
+        // the last segment starts from gs_out, an earlier one from the summaries of the pieces after it chained onto gs_out
+        float X[16];
+        bool have = false;
+        if (role < 3) {
+            if (seg == nseg - 1) {
+                have = gs_out != nullptr;
+                if (have) {
+                    const float *gp = gs_out + (size_t)bh * HEAD * HEAD;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int x = 16 * kk + 4 * g + e;
-                    G[kk][e] = role == 1 ? gp[own * HEAD + x] : gp[x * HEAD + own];
+                    for (int i = 0; i < 16; i++) {
+                        const int x = 16 * (i >> 2) + 4 * g + (i & 3);
+                        X[i] = role == 2 ? gp[x * HEAD + own] : gp[own * HEAD + x];
+                    }
                 }
+            } else {
+                int ki[16], vi[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int x = 16 * (i >> 2) + 4 * g + (i & 3);
+                    ki[i] = role == 2 ? x : own;
+                    vi[i] = role == 2 ? own : x;
+                }
+                const float *pcs = gpart + (size_t)bh * nseg * m * PART, *ends = gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr;
+                if (role == 2) chain_summaries<16, false>(X, ki, vi, pcs, (seg + 1) * m, (nseg - 1 - seg) * m, 1, ends);
+                else chain_summaries<16, true>(X, ki, vi, pcs, (seg + 1) * m, (nseg - 1 - seg) * m, 1, ends);
+                have = true;
+            }
+        }
+        if (have && (role == 1 || role == 2)) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) G[i >> 2][i & 3] = X[i];
         }
         if (role == 0) {       // anchor of the decay-gradient sum at the segment's end: sum_j G o S
             float a = 0.f;
-            if (gp) {
+            if (have) {
                 const float *cp = ck_lane + (size_t)sb1 * HEAD * HEAD;
 #pragma unroll
-                for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) a = fmaf(gp[own * HEAD + 16 * kk + 4 * g + e], cp[kk * 1024 + e * 4], a);
+                for (int i = 0; i < 16; i++) a = fmaf(X[i], cp[(i >> 2) * 1024 + (i & 3) * 4], a);
             }
             a = group_sum4(a);
             if (g == 0) sm.arun[0][own] = a;
@@ -1186,39 +1302,6 @@ __global__ void sum_partials(int B, int H, int nA, int nseg, const float *__rest
     out[c] = sum;
 }
 
-// Chains the piece summaries (S_out = decay o S_in + delta, one decay per key) of one
-// (batch, head) in order, one lane per state element.  `first`..`last` are the pieces
-// the pass produced; going up (forward, step = +1) it starts from `start` and leaves
-// the state at the start of segment s in the slot of piece s*m - 1; going down
-// (backward, step = -1) it leaves the gradient at the end of segment s in the slot of
-// piece (s+1)*m.  In place: a slot is overwritten by the lane that has just read it.
-__global__ __launch_bounds__(256) void fold_summaries(int bh0, int first, int last, int step, int m, int stride,
-        const float *__restrict__ start, float *__restrict__ part)
-{
-    const int bh = bh0 + blockIdx.x / (HEAD * HEAD / 256), el = (blockIdx.x % (HEAD * HEAD / 256)) * 256 + threadIdx.x;
-    const int key = el / HEAD;
-    float *pp = part + (size_t)bh * stride * PART;
-    float S = start ? start[(size_t)bh * HEAD * HEAD + el] : 0.f;
-    const int count = (last - first) * step + 1;
-    for (int i0 = 0; i0 < count; i0 += 4) {        // four loads in flight per lane
-        float dl[4], dd[4];
-#pragma unroll
-        for (int x = 0; x < 4; x++)
-            if (i0 + x < count) {
-                const float *q = pp + (size_t)(first + (i0 + x) * step) * PART;
-                dl[x] = q[el];
-                dd[x] = q[HEAD * HEAD + key];
-            }
-#pragma unroll
-        for (int x = 0; x < 4; x++)
-            if (i0 + x < count) {
-                const int piece = first + (i0 + x) * step;
-                S = fmaf(dd[x], S, dl[x]);
-                if (step > 0 ? (piece + 1) % m == 0 : piece % m == 0) pp[(size_t)piece * PART + el] = S;
-            }
-    }
-}
-
 // ------------------------------------------------------------------ launchers --
 size_t checkpoint_bytes(int B, int Tlen, int H) {
     return (size_t)B * H * ((Tlen + SB - 1) / SB + 1) * HEAD * HEAD * sizeof(float);     // one slot per step + the final state
@@ -1323,8 +1406,7 @@ hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tl
     const SegPlan &pl = gp.b;
     const int nB = BH - gp.nA;
     if (pl.nseg > 1) {
-        const int pieces = (pl.nseg - 1) * pl.m;
-        dim3 grid(nB * pieces), block(NT_F);
+        dim3 grid(nB * (pl.nseg - 1) * pl.m), block(NT_F);
         if (mode == 2)
             hipLaunchKernelGGL((summary_pass<true, false, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
                                pl.pps, kk, vv, w, part, floor_decay);
@@ -1334,8 +1416,6 @@ hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tl
         else
             hipLaunchKernelGGL((summary_pass<false, false, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
                                pl.pps, kk, vv, w, part, floor_decay);
-        hipLaunchKernelGGL(fold_summaries, dim3(nB * (HEAD * HEAD / 256)), dim3(256), 0, s, gp.nA, 0, pieces - 1, 1, pl.m,
-                           pl.nseg * pl.m, s_in, part);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -1387,8 +1467,7 @@ hipError_t backward_launch(hipStream_t s, bool per_token, bool w16, int B, int T
     const int nB = BH - gp.nA;
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v, *gg = (const bf16 *)gy;
     if (pl.nseg > 1) {
-        const int pieces = (pl.nseg - 1) * pl.m;
-        dim3 grid(nB * pieces), block(NT_F);
+        dim3 grid(nB * (pl.nseg - 1) * pl.m), block(NT_F);
         if (mode == 2)
             hipLaunchKernelGGL((summary_pass<true, true, true>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
                                pl.pps, rr, gg, w, gpart, floor_decay);
@@ -1398,8 +1477,6 @@ hipError_t backward_launch(hipStream_t s, bool per_token, bool w16, int B, int T
         else
             hipLaunchKernelGGL((summary_pass<false, true, false>), grid, block, 0, s, gp.nA, Tlen, C, H, pl.nseg, pl.sps, pl.m,
                                pl.pps, rr, gg, w, gpart, floor_decay);
-        hipLaunchKernelGGL(fold_summaries, dim3(nB * (HEAD * HEAD / 256)), dim3(256), 0, s, gp.nA, pl.nseg * pl.m - 1, pl.m,
-                           -1, pl.m, pl.nseg * pl.m, gs_out, gpart);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
