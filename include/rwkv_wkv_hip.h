@@ -64,10 +64,19 @@ typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
 const char *wkv_strerror(int status);
 int wkv_abi_version(void);
 
+/* One-time set-up of the loaded kernels on the current process (raises the LDS limit of the blocked kernels; no
+ * counterpart in the reference, whose extension is configured when torch builds it, RWKV-v5/src/module/TimeMix.py:
+ * 229-252).  The operators do it themselves on their first call; call it once beforehand when that first call
+ * would fall inside a HIP stream capture.  Needs a GPU; returns WKV_ERR_LAUNCH without one. */
+int wkv_init(void);
+
 /* Tuning knobs (no counterpart in the reference).  WKV_TUNE_SEGMENTS: number of
  * time segments one (batch, head) sequence is cut into by the chunked algorithm
  * so that short batches still fill the GPU; 0 = choose from the shape (default),
- * 1..64 = force.  Results do not depend on it beyond fp32 rounding order. */
+ * 1..64 = force.  Results do not depend on it beyond fp32 rounding order.  The workspace sizes the queries return
+ * depend on it (more segments, more piece summaries): query again after changing it.  It may change between a
+ * forward call and its backward call (only the state checkpoints pass between the two, and those do not depend
+ * on it). */
 #define WKV_TUNE_SEGMENTS 1
 int wkv_tune(int key, int value);
 

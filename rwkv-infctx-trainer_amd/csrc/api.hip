@@ -58,7 +58,7 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
             if (workspace_bytes < chunked::forward_workspace(B, T, H)) return WKV_ERR_WORKSPACE;
         }
         hipError_t e = chunked::forward_launch((hipStream_t)stream, per_token, w16, B, T, C, H, r, k, v, w, u, state_in, y,
-                                               state_out, workspace, true, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+                                               state_out, workspace, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
         return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
     }
     hipError_t e = recurrent_forward((hipStream_t)stream, dtype, per_token, B, T, C, H, r, k, v, (const float *)w, u, state_in, y,
@@ -137,7 +137,9 @@ const char *wkv_strerror(int status) {
     }
 }
 
-int wkv_abi_version(void) { return 1; }
+int wkv_abi_version(void) { return 2; }
+
+int wkv_init(void) { return chunked::init_kernels() == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH; }
 
 int wkv_tune(int key, int value) {
     if (key == WKV_TUNE_SEGMENTS) {

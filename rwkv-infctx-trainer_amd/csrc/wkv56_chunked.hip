@@ -1303,13 +1303,28 @@ __global__ void sum_partials(int B, int H, int nA, int nseg, const float *__rest
 }
 
 // ------------------------------------------------------------------ launchers --
+static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t checkpoint_bytes(int B, int Tlen, int H) {
     return (size_t)B * H * ((Tlen + SB - 1) / SB + 1) * HEAD * HEAD * sizeof(float);     // one slot per step + the final state
 }
 
+// Compute units of the current device (256 on MI355X; also the answer when no device can be asked, as in a
+// workspace query made on a machine without one).
+static int cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 256; }
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) { (void)hipGetLastError(); n = 256; }
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 // How many time segments run in parallel for one (batch, head).  More segments mean
-// more workgroups (B*H*nseg) to spread over the 256 CUs but also one more light pass
-// over the inputs and a longer fold; the estimate below counts CU rounds times steps
+// more workgroups (B*H*nseg) to spread over the compute units but also one more light pass
+// over (part of) the inputs; the estimate below counts CU rounds times steps
 // per segment and prefers fewer segments on ties.  wkv_tune(WKV_TUNE_SEGMENTS) /
 // RWKV_WKV_NSEG override it.
 constexpr int MAX_SEG = 64;
@@ -1322,10 +1337,10 @@ inline int &forced_piece_steps() {       // 0 = choose automatically
     static int v = [] { const char *e = getenv("RWKV_WKV_PPS"); return e ? std::max(atoi(e), 0) : 0; }();
     return v;
 }
-// what the summary pass and the fold add to a run in n segments, as a factor on the main kernels' time
-// (the pass reads (n-1)/n of the tokens at about 40 % of the main kernels' cost per token)
+// what the summary pass adds to a run in n segments, as a factor on the main kernels' time
+// (at worst the pass reads (n-1)/n of the tokens at about 40 % of the main kernels' cost per token)
 static double segment_overhead(int n) { return 1.0 + 0.4 * (n - 1) / n; }
-static SegPlan plan_segments(int BH, int Tlen) {
+static SegPlan plan_segments(int BH, int Tlen, int ncu) {
     const int nsb = (Tlen + SB - 1) / SB;
     const int forced = forced_segments();
     int want = 1;
@@ -1335,7 +1350,7 @@ static SegPlan plan_segments(int BH, int Tlen) {
         double best = 1e30;
         for (int cand = 1; cand <= 16 && cand * 4 <= std::max(4, nsb); cand++) {
             const int sps = (nsb + cand - 1) / cand;
-            const double rounds = (double)((BH * cand + 255) / 256);
+            const double rounds = (double)((BH * cand + ncu - 1) / ncu);
             const double cost = rounds * (sps + 1) * segment_overhead(cand);
             if (cost < best * 0.97) { best = cost; want = cand; }
         }
@@ -1343,14 +1358,15 @@ static SegPlan plan_segments(int BH, int Tlen) {
     const int sps = (nsb + want - 1) / want;
     const int nseg = (nsb + sps - 1) / sps;
     // the summary pass: cut each segment into pieces until the pass has about 1.5 workgroups per CU
-    // (every piece costs one 16 KB summary and a step of the fold, so no finer than needed and never below 2 steps)
+    // (every piece costs one 16 KB summary, so no finer than needed and never below 2 steps)
     int pps = sps;
     if (nseg == 1) return SegPlan{1, sps, 1, sps};
     if (forced_piece_steps() > 0) pps = std::min(sps, forced_piece_steps());
     else
-        while (pps >= 4 && (long)BH * (nseg - 1) * ((sps + pps - 1) / pps) < 384) pps = (pps + 1) / 2;
+        while (pps >= 4 && (long)BH * (nseg - 1) * ((sps + pps - 1) / pps) < ncu + ncu / 2) pps = (pps + 1) / 2;
     int m = (sps + pps - 1) / pps;
     if (nseg * m > MAX_SEG) { m = std::max(1, MAX_SEG / nseg); pps = (sps + m - 1) / m; m = (sps + pps - 1) / pps; }
+    if (nseg * m > MAX_SEG) { m = 1; pps = sps; }
     return SegPlan{nseg, sps, m, pps};
 }
 // Two groups of (batch, head) pairs.  When B*H is more than a whole number of CU rounds, the whole rounds run their
@@ -1358,50 +1374,69 @@ static SegPlan plan_segments(int BH, int Tlen) {
 // (group B), so that it fills one more, shorter round: 320 pairs = 256 whole + 64 x 4 segments instead of 320 x 4.
 struct GroupPlan { int nA; SegPlan a, b; };
 static GroupPlan plan_groups(int BH, int Tlen) {
-    const int nsb = (Tlen + SB - 1) / SB;
-    GroupPlan p{0, SegPlan{1, nsb, 1, nsb}, plan_segments(BH, Tlen)};
-    const int whole = BH / 256 * 256, rest = BH - whole;
+    const int nsb = (Tlen + SB - 1) / SB, ncu = cu_count();
+    GroupPlan p{0, SegPlan{1, nsb, 1, nsb}, plan_segments(BH, Tlen, ncu)};
+    const int whole = BH / ncu * ncu, rest = BH - whole;
     if (forced_segments() > 0 || whole == 0 || rest == 0) return p;
-    const SegPlan r = plan_segments(rest, Tlen);
-    auto cost = [](int bh, const SegPlan &x) {
-        return (double)((bh * x.nseg + 255) / 256) * (x.sps + 1) * segment_overhead(x.nseg);
+    const SegPlan r = plan_segments(rest, Tlen, ncu);
+    auto cost = [ncu](int bh, const SegPlan &x) {
+        return (double)((bh * x.nseg + ncu - 1) / ncu) * (x.sps + 1) * segment_overhead(x.nseg);
     };
     if (cost(whole, p.a) + cost(rest, r) < 0.97 * cost(BH, p.b)) { p.nA = whole; p.b = r; }
     return p;
 }
-static size_t part_bytes(int B, int H) { return (size_t)B * H * MAX_SEG * PART * sizeof(float); }
-
-// workspace of a forward call: checkpoints | forward segment summaries
-size_t forward_workspace(int B, int Tlen, int H) { return checkpoint_bytes(B, Tlen, H) + part_bytes(B, H); }
-// workspace of a backward call: the forward's | backward segment summaries | gu, gw partials, each (B, C) for the
-// unsplit group and (B*MAX_SEG, C) for the split one
-size_t backward_workspace(int B, int Tlen, int C, int H) {
-    return forward_workspace(B, Tlen, H) + part_bytes(B, H) + 2 * (size_t)B * (MAX_SEG + 1) * C * sizeof(float);
+// the piece summaries of a plan: one slot per (batch, head) and piece (slots are indexed by the pair's number in the
+// whole batch, so the pairs of group A have unused ones)
+static size_t part_bytes(int BH, const GroupPlan &gp) {
+    return gp.b.nseg > 1 ? round256((size_t)BH * gp.b.nseg * gp.b.m * PART * sizeof(float)) : 0;
 }
 
-template <class K>
-static hipError_t allow_lds(K kernel, size_t bytes) {
-    return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+// Where things are in a workspace, for the plan in force:  checkpoints | forward piece summaries | backward piece
+// summaries | gu, gw partial sums, each (B, C) for the unsplit group and (B*nseg, C) for the split one.  A forward
+// call uses the first two regions.  Only the checkpoints pass from a forward call to the backward call that follows,
+// and their place and layout depend on the shape alone, not on the plan.
+struct Layout { size_t ckpt, part, gpart, sums, forward_total, total; };
+static Layout layout(int B, int Tlen, int C, int H, const GroupPlan &gp) {
+    Layout L;
+    L.ckpt = 0;
+    L.part = round256(checkpoint_bytes(B, Tlen, H));
+    L.gpart = L.part + part_bytes(B * H, gp);
+    L.forward_total = L.gpart;
+    L.sums = L.gpart + part_bytes(B * H, gp);
+    L.total = L.sums + round256(2 * (size_t)B * (gp.b.nseg + 1) * C * sizeof(float));
+    return L;
+}
+size_t forward_workspace(int B, int Tlen, int H) { return layout(B, Tlen, H * HEAD, H, plan_groups(B * H, Tlen)).forward_total; }
+size_t backward_workspace(int B, int Tlen, int C, int H) { return layout(B, Tlen, C, H, plan_groups(B * H, Tlen)).total; }
+
+// The 16-wavefront kernels use more LDS than a kernel gets by default.  Raising the limit is a property of the loaded
+// code object and is done once, from wkv_init() or from the first launch, whichever comes first.
+hipError_t init_kernels() {
+    static hipError_t status = [] {
+        auto allow = [](const void *kernel, size_t bytes) {
+            return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        };
+        hipError_t e = allow((const void *)forward16<true, false>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)forward16<true, true>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)forward16<false, false>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)backward16<true, false>, sizeof(Bwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)backward16<true, true>, sizeof(Bwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)backward16<false, false>, sizeof(Bwd16Tiles));
+        return e;
+    }();
+    return status;
 }
 
-// workspace == nullptr: single segment, no checkpoints kept
+// ckpt == nullptr: no checkpoints kept;  part == nullptr: the sequences run in one piece each
 // w16: the per-token decay is bf16 (per_token only)
 hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tlen, int C, int H, const void *r, const void *k,
                           const void *v, const void *w, const float *u, const float *s_in, void *y, float *s_out,
-                          void *workspace, bool keep_ckpt, int floor_decay) {
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = allow_lds(forward16<true, false>, sizeof(Fwd16Tiles));
-        if (e == hipSuccess) e = allow_lds(forward16<true, true>, sizeof(Fwd16Tiles));
-        if (e == hipSuccess) e = allow_lds(forward16<false, false>, sizeof(Fwd16Tiles));
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+                          float *ckpt, float *part, const GroupPlan &plan, int floor_decay) {
+    hipError_t e0 = init_kernels();
+    if (e0 != hipSuccess) return e0;
     const int mode = per_token ? (w16 ? 2 : 1) : 0;
     const int nsb = (Tlen + SB - 1) / SB, BH = B * H;
-    const GroupPlan gp = workspace ? plan_groups(BH, Tlen) : GroupPlan{0, SegPlan{1, nsb, 1, nsb}, SegPlan{1, nsb, 1, nsb}};
-    float *ckpt = (workspace && keep_ckpt) ? (float *)workspace : nullptr;
-    float *part = workspace ? (float *)((char *)workspace + checkpoint_bytes(B, Tlen, H)) : nullptr;
+    const GroupPlan gp = part ? plan : GroupPlan{0, SegPlan{1, nsb, 1, nsb}, SegPlan{1, nsb, 1, nsb}};
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v;
     const SegPlan &pl = gp.b;
     const int nB = BH - gp.nA;
@@ -1440,30 +1475,36 @@ hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tl
     return hipGetLastError();
 }
 
+// forward with a caller's workspace (or none: one piece per sequence, no checkpoints)
+hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tlen, int C, int H, const void *r, const void *k,
+                          const void *v, const void *w, const float *u, const float *s_in, void *y, float *s_out,
+                          void *workspace, int floor_decay) {
+    const GroupPlan gp = plan_groups(B * H, Tlen);
+    const Layout L = layout(B, Tlen, C, H, gp);
+    char *ws = (char *)workspace;
+    return forward_launch(s, per_token, w16, B, Tlen, C, H, r, k, v, w, u, s_in, y, s_out, ws ? (float *)(ws + L.ckpt) : nullptr,
+                          (ws && gp.b.nseg > 1) ? (float *)(ws + L.part) : nullptr, gp, floor_decay);
+}
+
 hipError_t backward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tlen, int C, int H, const void *r, const void *k,
                            const void *v, const void *w, const float *u, const float *s_in, const void *gy,
                            const float *gs_out, void *gr, void *gk, void *gv, void *gw, float *gu, float *gs_in,
                            void *workspace, bool have_ckpt, int floor_decay) {
-    float *ckpt = (float *)workspace;
-    float *gpart = (float *)((char *)workspace + forward_workspace(B, Tlen, H));
-    float *gu_one = (float *)((char *)gpart + part_bytes(B, H)), *gu_many = gu_one + (size_t)B * C;
-    float *gw_one = gu_many + (size_t)B * MAX_SEG * C, *gw_many = gw_one + (size_t)B * C;
-    if (!have_ckpt) {      // the forward call did not leave its checkpoints here: rebuild them
-        hipError_t e = forward_launch(s, per_token, w16, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, workspace,
-                                      true, floor_decay);
-        if (e != hipSuccess) return e;
-    }
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = allow_lds(backward16<true, false>, sizeof(Bwd16Tiles));
-        if (e == hipSuccess) e = allow_lds(backward16<true, true>, sizeof(Bwd16Tiles));
-        if (e == hipSuccess) e = allow_lds(backward16<false, false>, sizeof(Bwd16Tiles));
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    hipError_t e0 = init_kernels();
+    if (e0 != hipSuccess) return e0;
     const int BH = B * H, mode = per_token ? (w16 ? 2 : 1) : 0;
     const GroupPlan gp = plan_groups(BH, Tlen);
+    const Layout L = layout(B, Tlen, C, H, gp);
     const SegPlan &pl = gp.b;
+    char *ws = (char *)workspace;
+    float *ckpt = (float *)(ws + L.ckpt), *gpart = (float *)(ws + L.gpart);
+    float *gu_one = (float *)(ws + L.sums), *gu_many = gu_one + (size_t)B * C;
+    float *gw_one = gu_many + (size_t)B * pl.nseg * C, *gw_many = gw_one + (size_t)B * C;
+    if (!have_ckpt) {      // the forward call did not leave its checkpoints here: rebuild them
+        hipError_t e = forward_launch(s, per_token, w16, B, Tlen, C, H, r, k, v, w, u, s_in, nullptr, nullptr, ckpt,
+                                      pl.nseg > 1 ? (float *)(ws + L.part) : nullptr, gp, floor_decay);
+        if (e != hipSuccess) return e;
+    }
     const int nB = BH - gp.nA;
     const bf16 *rr = (const bf16 *)r, *kk = (const bf16 *)k, *vv = (const bf16 *)v, *gg = (const bf16 *)gy;
     if (pl.nseg > 1) {

@@ -26,6 +26,7 @@ _I = c_int
 SIGNATURES = {
     "wkv_strerror": (c_char_p, [_I]),
     "wkv_abi_version": (_I, []),
+    "wkv_init": (_I, []),
     "wkv_tune": (_I, [_I, _I]),
     "wkv_profile_begin": (_I, [_I, _I]),
     "wkv_profile_end": (_I, [_P, _I]),
@@ -65,6 +66,12 @@ def lib():
             fn.restype = res
             fn.argtypes = args
         _lib = L
+        try:
+            import torch
+            if torch.cuda.is_available():
+                L.wkv_init()         # so that no operator call has set-up left to do (e.g. inside a graph capture)
+        except Exception:            # noqa: BLE001 - set-up then happens on the first call
+            pass
     return _lib
 
 

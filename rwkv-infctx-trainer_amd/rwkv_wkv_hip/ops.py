@@ -106,10 +106,11 @@ def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate, ws, alg
     if w32.dtype == torch.bfloat16:
         flags |= _lib.W_BF16           # gw comes back in bf16 too (torch.empty_like above)
     fn, wsq = (L.wkv5_backward, L.wkv5_backward_workspace) if version == 5 else (L.wkv6_backward, L.wkv6_backward_workspace)
-    if ws is not None:
+    need = wsq(B, T, C, H, dt, algo)
+    if ws is not None and ws.numel() >= need:
         flags |= _lib.CHECKPOINTS_VALID
-    else:
-        ws = _workspace(wsq(B, T, C, H, dt, algo), r.device)
+    else:           # no forward workspace, or one sized for another plan (wkv_tune changed in between): rebuild inside
+        ws = _workspace(need, r.device)
     check(fn(_stream(), B, T, C, H, dt, flags, algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
              _ptr(gy), _ptr(gstate), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs), _ptr(ws), ws.numel()),
           f"wkv{version}_backward")

@@ -35,7 +35,7 @@ def test_header_symbols_exported(L):
 
 
 def test_version_and_messages(L):
-    assert L.wkv_abi_version() == 1
+    assert L.wkv_abi_version() == 2
     assert L.wkv_strerror(0) == b"ok"
     for code in range(-8, 0):
         assert L.wkv_strerror(code) not in (b"ok", b"unknown status")

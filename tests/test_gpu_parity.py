@@ -418,3 +418,27 @@ def test_chunked_needs_the_decay_floor():
     y_ref, s_ref = O.wkv6_op(1, 1, 64, 1, t["r"], t["k"], t["v"], t["w"], t["u"], t["state"])
     assert_close(y, y_ref, 2e-2, "y")
     assert_close(s, s_ref, 1e-3, "state")
+
+
+@pytest.mark.parametrize("nseg_fwd,nseg_bwd", [(4, 2), (2, 8), (0, 3)])
+def test_plan_may_change_between_forward_and_backward(nseg_fwd, nseg_bwd):
+    """The number of time segments (wkv_tune) differs between the forward call and its backward call: only the
+    state checkpoints pass between the two, so every gradient still matches the oracle."""
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    wl = configs.make(3, B=1, T=1024, C=128, H=2, dtype=torch.bfloat16)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.to(dev()) for n, x in wl.tensors.items()}
+    leaves = {n: g[n].clone().requires_grad_(True) for n in ("r", "k", "v", "w", "u", "state")}
+    try:
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg_fwd) == 0
+        y, s = W.WKV_6.apply(B, T, C, H, leaves["r"], leaves["k"], leaves["v"], leaves["w"], leaves["u"], leaves["state"])
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg_bwd) == 0
+        torch.autograd.backward([y, s], [g["dy"], g["dstate"]])
+        torch.cuda.synchronize()
+    finally:
+        L.wkv_tune(_lib.TUNE_SEGMENTS, 0)
+    got = dict(y=y, state=s, gr=leaves["r"].grad, gk=leaves["k"].grad, gv=leaves["v"].grad, gw=leaves["w"].grad,
+               gu=leaves["u"].grad, gstate=leaves["state"].grad)
+    compare(got, run_oracle56(6, wl), 2e-2, f"plan {nseg_fwd}->{nseg_bwd}")
