@@ -115,6 +115,19 @@ int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned f
                  const float *state_in, void *y, float *state_out,
                  void *workspace, size_t workspace_bytes);
 
+/* wkv6_forward for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arguments and results as wkv6_forward with the chunked algorithm (bf16 r/k/v/y and WKV_FLOOR_DECAY required,
+ * else WKV_ERR_ALGO) and no state checkpoints kept; the scratch memory of the time-parallel split (the piece
+ * summaries) is a 16 MiB array inside the library, one per GPU, held until the process ends.  The call allocates
+ * nothing and frees nothing.  Shapes whose summaries exceed the array (B*H*segments*pieces*16640 bytes > 16 MiB,
+ * e.g. B*H above about 120 at T = 4096) are rejected with WKV_ERR_WORKSPACE.  All calls on one GPU share that
+ * GPU's array: two calls that overlap in time on the same GPU (different streams) race on it. */
+#define WKV_NOALLOC_SCRATCH_BYTES (16u << 20)
+int wkv6_forward_noalloc(void *stream, int B, int T, int C, int H, int dtype, unsigned flags,
+                         const void *r, const void *k, const void *v, const void *w, const float *u,
+                         const float *state_in, void *y, float *state_out);
+
 size_t wkv6_backward_workspace(int B, int T, int C, int H, int dtype, int algo);
 /* gstate_out may be NULL (no gradient arrives through the state handed out,
  * i.e. truncated BPTT); gstate_in may be NULL when it is not wanted. */

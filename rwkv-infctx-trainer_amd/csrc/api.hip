@@ -5,6 +5,7 @@
 #include "common.h"
 #include "wkv56_recurrent.hip"
 #include "wkv56_chunked.hip"
+#include "wkv56_noalloc.hip"
 #include "wkv4.hip"
 #include "cumsum_decay.hip"
 
@@ -197,6 +198,27 @@ int wkv5_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned f
                  float *state_out, void *workspace, size_t workspace_bytes) {
     return forward56(false, stream, B, T, C, H, dtype, flags, algo, r, k, v, w, u, state_in, y, state_out, workspace,
                      workspace_bytes);
+}
+
+int wkv6_forward_noalloc(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, const void *r,
+                         const void *k, const void *v, const void *w, const float *u, const float *state_in, void *y,
+                         float *state_out) {
+    int st = check_dims56(B, T, C, H, dtype);
+    if (st) return st;
+    if (!r || !k || !v || !w || !u || !state_in || !y || !state_out) return WKV_ERR_NULL;
+    for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
+                          (const void *)state_out})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    {
+        const uintptr_t a0 = reinterpret_cast<uintptr_t>(state_in), b0 = reinterpret_cast<uintptr_t>(state_out);
+        const size_t bytes = (size_t)B * H * HEAD * HEAD * sizeof(float);
+        if (a0 < b0 + bytes && b0 < a0 + bytes) return WKV_ERR_ALIAS;
+    }
+    if (pick_algo56(WKV_ALGO_CHUNKED, T, dtype, flags) != WKV_ALGO_CHUNKED) return WKV_ERR_ALGO;
+    hipError_t e = chunked::forward_static_launch((hipStream_t)stream, true, (flags & WKV_W_BF16) != 0, B, T, C, H, r, k, v, w,
+                                                  u, state_in, y, state_out, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
+    if (e == hipErrorOutOfMemory) return WKV_ERR_WORKSPACE;
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
 
 size_t wkv6_backward_workspace(int B, int T, int C, int H, int dtype, int algo) {

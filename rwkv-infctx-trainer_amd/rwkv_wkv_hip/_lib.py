@@ -32,6 +32,7 @@ SIGNATURES = {
     "wkv_profile_end": (_I, [_P, _I]),
     "wkv6_forward_workspace": (c_size_t, [_I] * 6),
     "wkv6_forward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 8 + [_P, c_size_t]),
+    "wkv6_forward_noalloc": (_I, [_P, _I, _I, _I, _I, _I, c_uint] + [_P] * 8),
     "wkv6_backward_workspace": (c_size_t, [_I] * 6),
     "wkv6_backward": (_I, [_P, _I, _I, _I, _I, _I, c_uint, _I] + [_P] * 14 + [_P, c_size_t]),
     "wkv5_forward_workspace": (c_size_t, [_I] * 6),
