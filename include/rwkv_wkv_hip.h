@@ -195,6 +195,18 @@ int wkv_cumsum_decay(void *stream, int Bw, int T, int C, int chunk_len, int per_
                      const float *w, float *log_w, float *incl, float *inter, float *intra,
                      float *chunk_sum);
 
+/* The same helper with every table the reference derives from w: besides the five log-space tables above,
+ *   ws_exp     (Bw,T/chunk,C) fp32  exp(chunk_sum)                        rwkv_inner.py:80
+ *   inter_exp  (Bw,T,C)       fp32  exp(inter)                            :81
+ *   intra_exp  (Bw,T,C)       fp32  exp(intra)                            :82
+ *   r_decay    (Bw,T,C)  exp(intra - intra at the chunk's token chunk_len/2)      :91-92
+ *   k_inv_decay(Bw,T,C)  exp(intra at the chunk's token chunk_len/2 - incl)       :91,93
+ * the last two in fp64 (precision = 64, double*) or fp32 (precision = 32, float*), as the reference's `precision`
+ * argument (:41-46): in fp32 they overflow for chunk lengths much beyond 32.  Any output pointer may be NULL. */
+int wkv_cumsum_decay_factors(void *stream, int Bw, int T, int C, int chunk_len, int per_token, int precision,
+                             const float *w, float *log_w, float *incl, float *inter, float *intra, float *chunk_sum,
+                             float *ws_exp, float *inter_exp, float *intra_exp, void *r_decay, void *k_inv_decay);
+
 #ifdef __cplusplus
 }
 #endif

@@ -285,4 +285,16 @@ int wkv_cumsum_decay(void *stream, int Bw, int T, int C, int chunk_len, int per_
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
 
+int wkv_cumsum_decay_factors(void *stream, int Bw, int T, int C, int chunk_len, int per_token, int precision,
+                             const float *w, float *log_w, float *incl, float *inter, float *intra, float *chunk_sum,
+                             float *ws_exp, float *inter_exp, float *intra_exp, void *r_decay, void *k_inv_decay) {
+    if (Bw <= 0 || T <= 0 || C <= 0 || chunk_len <= 0 || T % chunk_len != 0) return WKV_ERR_DIMS;
+    if (T / chunk_len > 65535 || Bw > 65535) return WKV_ERR_DIMS;
+    if (precision != 32 && precision != 64) return WKV_ERR_DTYPE;
+    if (!w) return WKV_ERR_NULL;
+    hipError_t e = cumsum_decay_factors_launch((hipStream_t)stream, Bw, T, C, chunk_len, per_token, precision, w, log_w, incl,
+                                               inter, intra, chunk_sum, ws_exp, inter_exp, intra_exp, r_decay, k_inv_decay);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
 }  // extern "C"

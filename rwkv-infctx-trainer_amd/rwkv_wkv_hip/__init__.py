@@ -1,7 +1,8 @@
 """MI355X-native WKV time-mix operators (RWKV v4 / v5 / v6) behind the
 reference trainer's autograd call signatures.  See ops.py."""
 from ._lib import WKVError, LIB_PATH
-from .ops import (WKV_5, WKV_6, RUN_WKV5_CUDA, RUN_WKV6STATE_CUDA, wkv_op, cumsum_decay, set_algo)
+from .ops import (WKV_5, WKV_6, RUN_WKV5_CUDA, RUN_WKV6STATE_CUDA, wkv_op, cumsum_decay, set_algo, RecomputeCache,
+                  recompute_cache, stats)
 
 # the reference's class names, same in-place calling convention as its RUN_* wrappers
 class WKV5_CUDA:
@@ -13,4 +14,4 @@ class WKV6STATE_CUDA:
 
 
 __all__ = ["WKV_5", "WKV_6", "WKV5_CUDA", "WKV6STATE_CUDA", "RUN_WKV5_CUDA", "RUN_WKV6STATE_CUDA", "wkv_op",
-           "cumsum_decay", "set_algo", "WKVError", "LIB_PATH"]
+           "cumsum_decay", "set_algo", "RecomputeCache", "recompute_cache", "stats", "WKVError", "LIB_PATH"]

@@ -44,6 +44,7 @@ SIGNATURES = {
     "wkv4_backward_workspace": (c_size_t, [_I] * 4),
     "wkv4_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, c_size_t]),
     "wkv_cumsum_decay": (_I, [_P, _I, _I, _I, _I, _I] + [_P] * 6),
+    "wkv_cumsum_decay_factors": (_I, [_P, _I, _I, _I, _I, _I, _I] + [_P] * 11),
 }
 
 _lib = None

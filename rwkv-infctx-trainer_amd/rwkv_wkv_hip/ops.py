@@ -71,7 +71,81 @@ def _blocked(version, B, T, C, H, dtype):
     return T > 1 and dtype in _DT and fq(B, T, C, H, _DT[dtype], _algo) > 0
 
 
-def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad):
+stats = {"forward_launches": 0, "forward_reused": 0}      # counters for tests and diagnostics
+
+
+class RecomputeCache:
+    """Opt-in reuse of a forward pass by the recomputation that activation checkpointing runs later.
+
+    Under activation checkpointing (the reference wraps every block in ``deepspeed.checkpointing.checkpoint``,
+    RWKV-v5/src/model.py:674-683) the operator's forward runs twice per layer and segment: once without autograd
+    while the model runs forward, once more when backward recomputes the block.  With a cache installed
+    (``with recompute_cache(): ...`` around the training step) the first run keeps its outputs and its state
+    checkpoints, and the recomputation, which replays the blocks in reverse order, takes them over instead of
+    running the kernels again: one forward pass of the operator less per layer and segment, paid for with y, the new
+    state and the checkpoints (about 6 bytes per token and channel) held from forward to backward.
+
+    Matching is by order (last kept, first reused) and by signature (operator, shape, dtypes): it relies on the
+    recomputation replaying exactly the calls of the first run, as activation checkpointing does.  Forward runs
+    that are never recomputed (validation, generation) must stay outside the ``with`` block."""
+
+    def __init__(self, max_entries: int = 4096):
+        self.stack, self.max_entries = [], max_entries
+
+    def push(self, sig, payload):
+        if len(self.stack) >= self.max_entries:
+            self.stack.pop(0)
+        self.stack.append((sig, payload))
+
+    def pop(self, sig):
+        if self.stack and self.stack[-1][0] == sig:
+            return self.stack.pop()[1]
+        return None
+
+
+_cache = None
+
+
+class recompute_cache:
+    """Context manager that installs a ``RecomputeCache`` for the operators called inside it."""
+
+    def __init__(self, cache: RecomputeCache = None):
+        self.cache = cache or RecomputeCache()
+
+    def __enter__(self):
+        global _cache
+        self.prev, _cache = _cache, self.cache
+        return self.cache
+
+    def __exit__(self, *exc):
+        global _cache
+        _cache = self.prev
+        self.cache.stack.clear()
+        return False
+
+
+def _forward56_cached(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad, out_state=None):
+    """_forward56 behind the recompute cache (when one is installed)."""
+    cache = _cache
+    if cache is None:
+        return _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad, out_state)
+    sig = (version, B, T, C, H, r.dtype, w32.dtype, tuple(w32.shape))
+    if need_grad:
+        hit = cache.pop(sig)
+        if hit is not None:          # the recomputation of a forward run that kept its results
+            y, new_state, ws, algo = hit
+            if out_state is not None:
+                out_state.copy_(new_state)
+                new_state = out_state
+            stats["forward_reused"] += 1
+            return y, new_state, ws, algo
+        return _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, True, out_state)
+    y, new_state, ws, algo = _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, True, out_state)    # keep checkpoints
+    cache.push(sig, (y, new_state.clone() if out_state is not None else new_state, ws, algo))
+    return y, new_state, ws, algo
+
+
+def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad, out_state=None):
     """Returns y, new_state and, when a backward call will follow, the
     workspace in which the forward kernel left its state checkpoints (sized
     for that backward call) together with the algorithm that was in force.
@@ -80,7 +154,7 @@ def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad):
     dt = _check_rkv(B, T, C, H, r, k, v)
     _on_gpu(r, k, v, w32, u32, s32)
     y = torch.empty_like(r)
-    new_state = torch.empty_like(s32)
+    new_state = torch.empty_like(s32) if out_state is None else out_state       # (must not overlap s32)
     flags = _lib.FLOOR_DECAY if T > 1 else 0
     if w32.dtype == torch.bfloat16:
         flags |= _lib.W_BF16
@@ -92,6 +166,7 @@ def _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad):
         ws = _workspace(max(fq(B, T, C, H, dt, algo), bq(B, T, C, H, dt, algo)), r.device)
     check(fn(_stream(), B, T, C, H, dt, flags, algo, _ptr(r), _ptr(k), _ptr(v), _ptr(w32), _ptr(u32), _ptr(s32),
              _ptr(y), _ptr(new_state), _ptr(ws), 0 if ws is None else ws.numel()), f"wkv{version}_forward")
+    stats["forward_launches"] += 1
     return y, new_state, ws, algo
 
 
@@ -117,20 +192,17 @@ def _backward56(version, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate, ws, alg
     return gr, gk, gv, gw, gu, gs
 
 
-class WKV_5(torch.autograd.Function):
-    """WKV5: per-channel decay.  state (B,H,64,64) fp32 [key][value]; r,k,v
-    (B,T,C) in one dtype; w (H,64) fp32 raw; u (H,64)."""
-
+class _WKV5Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, B, T, C, H, state, r, k, v, w, u):
+    def forward(ctx, grad_mode, B, T, C, H, state, r, k, v, w, u):
         assert state.dtype == torch.float32 and w.dtype == torch.float32
         assert state.is_contiguous() and w.is_contiguous() and u.is_contiguous()
         assert state.shape == (B, H, HEAD, HEAD) and H * HEAD == C
         u32 = u.float().contiguous().view(H, HEAD)
         w32 = w.view(H, HEAD)
-        need_grad = any(ctx.needs_input_grad)        # all False under torch.no_grad(): no checkpoints kept then
+        need_grad = grad_mode and any(ctx.needs_input_grad)      # no checkpoints kept under torch.no_grad()
         with torch.no_grad():
-            y, new_state, ws, algo = _forward56(5, B, T, C, H, r, k, v, w32, u32, state, need_grad)
+            y, new_state, ws, algo = _forward56_cached(5, B, T, C, H, r, k, v, w32, u32, state, need_grad)
         ctx.dims = (B, T, C, H)
         ctx.meta = (w.shape, u.shape, u.dtype)
         ctx.ws, ctx.algo = ws, algo
@@ -147,26 +219,32 @@ class WKV_5(torch.autograd.Function):
         gstate = None if gstate is None else gstate.float().contiguous()
         with torch.no_grad():
             gr, gk, gv, gw, gu, gs = _backward56(5, B, T, C, H, r, k, v, w32, u32, state, gy, gstate, ctx.ws, ctx.algo)
-        return (None, None, None, None, gs, gr, gk, gv, gw.view(wshape), gu.view(ushape).to(udtype))
+        return (None, None, None, None, None, gs, gr, gk, gv, gw.view(wshape), gu.view(ushape).to(udtype))
 
 
-class WKV_6(torch.autograd.Function):
-    """WKV6: per-token decay.  r,k,v (B,T,C); w (B,T,C) raw (any float dtype,
-    used in fp32; a bf16 w is read as it is by the blocked algorithm and its
-    gradient comes back in bf16, as in the reference, RWKV-v6/src/module/
-    TimeMix.py:50,90); u (H,64); s (B,H,64,64) [key][value]."""
+class WKV_5:
+    """WKV5: per-channel decay.  ``WKV_5.apply(B, T, C, H, state, r, k, v, w, u) -> (y, new_state)`` with state
+    (B,H,64,64) fp32 [key][value]; r,k,v (B,T,C) in one dtype; w (H,64) fp32 raw; u (H,64).  Differentiable in
+    everything, the state included.  (A thin front of the autograd Function: it notes whether autograd is recording,
+    which the Function itself cannot see, so that a call under torch.no_grad() keeps no checkpoints.)"""
 
     @staticmethod
-    def forward(ctx, B, T, C, H, r, k, v, w, u, s):
+    def apply(B, T, C, H, state, r, k, v, w, u):
+        return _WKV5Fn.apply(torch.is_grad_enabled(), B, T, C, H, state, r, k, v, w, u)
+
+
+class _WKV6Fn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, grad_mode, B, T, C, H, r, k, v, w, u, s):
         assert s.is_contiguous() and w.is_contiguous() and u.is_contiguous()
         assert s.shape == (B, H, HEAD, HEAD) and H * HEAD == C and w.shape == (B, T, C)
         u32 = u.float().contiguous().view(H, HEAD)
         native_w = w.dtype == torch.bfloat16 and r.dtype == torch.bfloat16 and _blocked(6, B, T, C, H, r.dtype)
         w32 = w if native_w else w.float()
         s32 = s.float()
-        need_grad = any(ctx.needs_input_grad)
+        need_grad = grad_mode and any(ctx.needs_input_grad)
         with torch.no_grad():
-            y, new_state, ws, algo = _forward56(6, B, T, C, H, r, k, v, w32, u32, s32, need_grad)
+            y, new_state, ws, algo = _forward56_cached(6, B, T, C, H, r, k, v, w32, u32, s32, need_grad)
         ctx.dims = (B, T, C, H)
         ctx.meta = (w.dtype, u.shape, u.dtype, s.dtype)
         ctx.ws, ctx.algo = ws, algo
@@ -183,14 +261,83 @@ class WKV_6(torch.autograd.Function):
         gstate = None if gstate is None else gstate.float().contiguous()
         with torch.no_grad():
             gr, gk, gv, gw, gu, gs = _backward56(6, B, T, C, H, r, k, v, w32, u32, s32, gy, gstate, ctx.ws, ctx.algo)
-        return (None, None, None, None, gr, gk, gv, gw.to(wdtype), gu.view(ushape).to(udtype), gs.to(sdtype))
+        return (None, None, None, None, None, gr, gk, gv, gw.to(wdtype), gu.view(ushape).to(udtype), gs.to(sdtype))
+
+
+class WKV_6:
+    """WKV6: per-token decay.  ``WKV_6.apply(B, T, C, H, r, k, v, w, u, s) -> (y, new_state)`` with r,k,v (B,T,C);
+    w (B,T,C) raw (any float dtype, used in fp32; a bf16 w is read as it is by the blocked algorithm and its
+    gradient comes back in bf16, as in the reference, RWKV-v6/src/module/TimeMix.py:50,90); u (H,64);
+    s (B,H,64,64) [key][value]."""
+
+    @staticmethod
+    def apply(B, T, C, H, r, k, v, w, u, s):
+        return _WKV6Fn.apply(torch.is_grad_enabled(), B, T, C, H, r, k, v, w, u, s)
+
+
+class _RunInPlace5(torch.autograd.Function):
+    """WKV5 with the reference's in-place state convention: y is returned, the new state is written by the kernel
+    straight into the caller's buffer (e.g. one layer's slice of the trainer's (N_layer,B,H,64,64) tensor,
+    RWKV-v5/src/model.py:53-61), the incoming state survives in a private copy for backward (the reference's
+    ``state.clone()``, TimeMix.py:60).  No gradient flows through the state, as in the reference (:139-140)."""
+
+    @staticmethod
+    def forward(ctx, grad_mode, B, T, C, H, state, r, k, v, w, u):
+        u32, w32 = u.float().contiguous().view(H, HEAD), w.view(H, HEAD)
+        s_in = state.clone()
+        with torch.no_grad():
+            y, _, ws, algo = _forward56_cached(5, B, T, C, H, r, k, v, w32, u32, s_in, grad_mode and any(ctx.needs_input_grad),
+                                               out_state=state)
+        ctx.dims, ctx.meta, ctx.ws, ctx.algo = (B, T, C, H), (w.shape, u.shape, u.dtype), ws, algo
+        ctx.save_for_backward(r, k, v, w32, u32, s_in)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        B, T, C, H = ctx.dims
+        r, k, v, w32, u32, s_in = ctx.saved_tensors
+        wshape, ushape, udtype = ctx.meta
+        with torch.no_grad():
+            gr, gk, gv, gw, gu, _ = _backward56(5, B, T, C, H, r, k, v, w32, u32, s_in, gy.contiguous(), None, ctx.ws, ctx.algo)
+        return (None, None, None, None, None, None, gr, gk, gv, gw.view(wshape), gu.view(ushape).to(udtype))
+
+
+class _RunInPlace6(torch.autograd.Function):
+    """WKV6 counterpart of ``_RunInPlace5`` (RWKV-v6/src/module/TimeMix.py:51,111-118)."""
+
+    @staticmethod
+    def forward(ctx, grad_mode, B, T, C, H, r, k, v, w, u, s):
+        u32 = u.float().contiguous().view(H, HEAD)
+        native_w = w.dtype == torch.bfloat16 and r.dtype == torch.bfloat16 and _blocked(6, B, T, C, H, r.dtype)
+        w32 = w if native_w else w.float()
+        s_in = s.clone()
+        with torch.no_grad():
+            y, _, ws, algo = _forward56_cached(6, B, T, C, H, r, k, v, w32, u32, s_in, grad_mode and any(ctx.needs_input_grad),
+                                               out_state=s)
+        ctx.dims, ctx.meta, ctx.ws, ctx.algo = (B, T, C, H), (w.dtype, u.shape, u.dtype), ws, algo
+        ctx.save_for_backward(r, k, v, w32, u32, s_in)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        B, T, C, H = ctx.dims
+        r, k, v, w32, u32, s_in = ctx.saved_tensors
+        wdtype, ushape, udtype = ctx.meta
+        with torch.no_grad():
+            gr, gk, gv, gw, gu, _ = _backward56(6, B, T, C, H, r, k, v, w32, u32, s_in, gy.contiguous(), None, ctx.ws, ctx.algo)
+        return (None, None, None, None, None, gr, gk, gv, gw.to(wdtype), gu.view(ushape).to(udtype), None)
+
+
+def _direct_state(state, B, H):
+    return state.dtype == torch.float32 and state.is_contiguous() and state.shape == (B, H, HEAD, HEAD) and not state.requires_grad
 
 
 def RUN_WKV5_CUDA(B, T, C, H, state, r, k, v, w, u):
-    """The reference's calling convention (RWKV-v5/src/module/TimeMix.py:145-154):
-    returns y and leaves the new state in ``state``.  The operator works on a copy
-    of the incoming state, as the reference saves ``state.clone()`` (:60): the
-    tensor kept for backward must not be the one overwritten here."""
+    """The reference's calling convention (RWKV-v5/src/module/TimeMix.py:145-154): returns y and leaves the new
+    state in ``state``.  An fp32 contiguous state buffer is written by the kernel directly (no copy afterwards);
+    anything else goes through the functional operator and a copy."""
+    if _direct_state(state, B, H) and w.dtype == torch.float32 and w.is_contiguous() and u.is_contiguous():
+        return _RunInPlace5.apply(torch.is_grad_enabled(), B, T, C, H, state, r, k, v, w, u)
     y, new_state = WKV_5.apply(B, T, C, H, state.clone(), r, k, v, w, u)
     with torch.no_grad():
         state.copy_(new_state)
@@ -198,9 +345,10 @@ def RUN_WKV5_CUDA(B, T, C, H, state, r, k, v, w, u):
 
 
 def RUN_WKV6STATE_CUDA(B, T, C, H, r, k, v, w, u, s):
-    """The reference's calling convention (RWKV-v6/src/module/TimeMix.py:111-118):
-    returns y and leaves the new state in ``s`` (the operator works on a copy of
-    the incoming state, as the reference saves ``s.clone()``, :51)."""
+    """The reference's calling convention (RWKV-v6/src/module/TimeMix.py:111-118): returns y and leaves the new
+    state in ``s`` (written by the kernel directly when ``s`` is an fp32 contiguous buffer)."""
+    if _direct_state(s, B, H) and w.is_contiguous() and u.is_contiguous() and w.shape == (B, T, C):
+        return _RunInPlace6.apply(torch.is_grad_enabled(), B, T, C, H, r, k, v, w, u, s)
     y, new_state = WKV_6.apply(B, T, C, H, r, k, v, w, u, s.clone())
     with torch.no_grad():
         s.copy_(new_state)
@@ -209,7 +357,7 @@ def RUN_WKV6STATE_CUDA(B, T, C, H, r, k, v, w, u, s):
 
 class _WKV4(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, time_decay, time_first, k, v, wkv_state):
+    def forward(ctx, grad_mode, time_decay, time_first, k, v, wkv_state):
         L = _lib.lib()
         assert k.dim() == 3 and v.shape == k.shape and k.dtype == v.dtype
         B, T, C = k.shape
@@ -221,7 +369,7 @@ class _WKV4(torch.autograd.Function):
         k, v, st = k.contiguous(), v.contiguous(), wkv_state.float().contiguous()
         y = torch.empty_like(k)
         new_state = torch.empty_like(st)
-        need_grad = any(ctx.needs_input_grad)
+        need_grad = grad_mode and any(ctx.needs_input_grad)
         ckpt = _workspace(L.wkv4_checkpoint_bytes(B, T, C), k.device) if need_grad else None
         check(L.wkv4_forward(_stream(), B, T, C, _DT[k.dtype], _ptr(td), _ptr(tf), _ptr(k), _ptr(v), _ptr(st),
                              _ptr(y), _ptr(new_state), _ptr(ckpt)), "wkv4_forward")
@@ -243,20 +391,22 @@ class _WKV4(torch.autograd.Function):
         check(L.wkv4_backward(_stream(), B, T, C, _DT[k.dtype], _ptr(td), _ptr(tf), _ptr(k), _ptr(v), _ptr(st),
                               _ptr(gy), _ptr(gns), _ptr(gtd), _ptr(gtf), _ptr(gk), _ptr(gv), _ptr(gst), _ptr(ckpt),
                               _ptr(ws), ws.numel()), "wkv4_backward")
-        return gtd.to(ctx.meta[0]), gtf.to(ctx.meta[1]), gk, gv, gst
+        return None, gtd.to(ctx.meta[0]), gtf.to(ctx.meta[1]), gk, gv, gst
 
 
 def wkv_op(time_decay, time_first, k, v, wkv_state):
     """RWKV-v4 WKV with the signature of torch.ops.rwkv.wkv
     (RWKV-v4neo/src/model.py:130-132): time_decay, time_first (C); k, v (B,T,C);
     wkv_state (B,C,3) = (aa, bb, pp).  Returns (y, new_state)."""
-    return _WKV4.apply(time_decay, time_first, k, v, wkv_state)
+    return _WKV4.apply(torch.is_grad_enabled(), time_decay, time_first, k, v, wkv_state)
 
 
-def cumsum_decay(w, chunk_len=128, per_token=True):
-    """Log-space decay tables of the chunked formulation from the raw decay
-    parameter w (B,T,C) fp32, or (C,) expanded over T tokens when
-    ``per_token`` is an int T.  Returns dict(log_w, incl, inter, intra, chunk_sum)."""
+def cumsum_decay(w, chunk_len=128, per_token=True, factors=False, precision=64):
+    """Decay tables of the chunked formulation from the raw decay parameter w (B,T,C) fp32, or (C,) expanded over
+    T tokens when ``per_token`` is an int T.  Returns dict(log_w, incl, inter, intra, chunk_sum), all in log space;
+    with ``factors=True`` also the exponentiated tables ws_exp, inter_exp, intra_exp (fp32) and the two re-centred
+    factors r_decay, k_inv_decay of the intra-chunk product (fp64 for ``precision=64``, fp32 for 32), i.e.
+    everything RWKV-v5/src/module/rwkv_inner.py:43-93 derives from w."""
     L = _lib.lib()
     _on_gpu(w)
     w = w.float().contiguous()
@@ -265,8 +415,19 @@ def cumsum_decay(w, chunk_len=128, per_token=True):
         pt = 1
     else:
         (C,), Bw, T, pt = w.shape, 1, int(per_token), 0
-    out = {n: torch.empty(Bw, T, C, dtype=torch.float32, device=w.device) for n in ("log_w", "incl", "inter", "intra")}
+    new = lambda dt=torch.float32: torch.empty(Bw, T, C, dtype=dt, device=w.device)
+    out = {n: new() for n in ("log_w", "incl", "inter", "intra")}
     out["chunk_sum"] = torch.empty(Bw, T // chunk_len, C, dtype=torch.float32, device=w.device)
-    check(L.wkv_cumsum_decay(_stream(), Bw, T, C, chunk_len, pt, _ptr(w), _ptr(out["log_w"]), _ptr(out["incl"]),
-                             _ptr(out["inter"]), _ptr(out["intra"]), _ptr(out["chunk_sum"])), "wkv_cumsum_decay")
+    if not factors:
+        check(L.wkv_cumsum_decay(_stream(), Bw, T, C, chunk_len, pt, _ptr(w), _ptr(out["log_w"]), _ptr(out["incl"]),
+                                 _ptr(out["inter"]), _ptr(out["intra"]), _ptr(out["chunk_sum"])), "wkv_cumsum_decay")
+        return out
+    pdt = torch.float64 if precision == 64 else torch.float32
+    out["ws_exp"] = torch.empty_like(out["chunk_sum"])
+    out["inter_exp"], out["intra_exp"] = new(), new()
+    out["r_decay"], out["k_inv_decay"] = new(pdt), new(pdt)
+    check(L.wkv_cumsum_decay_factors(_stream(), Bw, T, C, chunk_len, pt, precision, _ptr(w), _ptr(out["log_w"]),
+                                     _ptr(out["incl"]), _ptr(out["inter"]), _ptr(out["intra"]), _ptr(out["chunk_sum"]),
+                                     _ptr(out["ws_exp"]), _ptr(out["inter_exp"]), _ptr(out["intra_exp"]),
+                                     _ptr(out["r_decay"]), _ptr(out["k_inv_decay"])), "wkv_cumsum_decay_factors")
     return out

@@ -230,6 +230,24 @@ def test_cumsum_decay_helper(chunk):
     cs = tab.chunk_log[..., 0, :].transpose(1, 2).reshape(B, T // chunk, C)
     assert_close(out["chunk_sum"], cs, 1e-5, "chunk_sum")
     assert out["log_w"][0, 9, 5].item() == pytest.approx(-5.298317, abs=1e-5)
+    # every table of the reference's helper, including the exponentiated ones and the re-centred fp64 factors
+    full = W.cumsum_decay(raw.to(dev()), chunk, factors=True, precision=64)
+    for n in ("log_w", "incl", "inter", "intra", "chunk_sum"):
+        assert torch.equal(full[n], out[n]), n
+    # (exponentials below the smallest normal fp32, 1.2e-38, come back as 0 from the GPU: absolute floor 1e-37; the
+    # exponents are fp32 sums of up to 128 terms of size ~5, summed in another order by torch: 2e-4 relative)
+    near = lambda a, b, n: torch.testing.assert_close(a.cpu(), b, rtol=2e-4, atol=1e-37, msg=lambda m: f"{n}: {m}")
+    near(full["ws_exp"], cs.exp(), "ws_exp")
+    near(full["inter_exp"], back(tab.inter_log).exp(), "inter_exp")
+    near(full["intra_exp"], back(tab.intra_log).exp(), "intra_exp")
+    assert full["r_decay"].dtype == torch.float64
+    lg = lambda x: x.double().log().float()          # compared in log space: the factors span hundreds of orders of magnitude
+    assert_close(lg(full["r_decay"].cpu()), lg(back(tab.r_decay)), 1e-5, "log r_decay")
+    assert_close(lg(full["k_inv_decay"].cpu()), lg(back(tab.k_inv_decay)), 1e-5, "log k_inv_decay")
+    if chunk == 16:
+        f32 = W.cumsum_decay(raw.to(dev()), chunk, factors=True, precision=32)
+        assert f32["r_decay"].dtype == torch.float32
+        assert_close(f32["r_decay"], back(O.cumsum_decay(w, chunk, 32).r_decay), 1e-4, "r_decay fp32")
     # per-channel (WKV5) form
     out5 = W.cumsum_decay(raw[0, 0].to(dev()), chunk, per_token=T)
     w5 = O.decay_from_raw(raw[0, 0]).view(1, H, 1, K).expand(1, H, T, K)

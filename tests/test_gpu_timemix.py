@@ -116,3 +116,26 @@ def test_in_place_wrappers_train(version):
     assert torch.equal(y, y2) and torch.equal(st, s2), "in-place wrapper and functional operator disagree"
     for n in names:
         assert torch.equal(La[n].grad, Lb[n].grad), f"gradient of {n} differs"
+
+
+@pytest.mark.parametrize("version", [5, 6])
+def test_in_place_wrappers_write_into_a_layer_slice(version):
+    """The state buffer handed to RUN_* is one layer's slice of an (N_layer, B, H, 64, 64) tensor, as the trainer keeps
+    it: the kernel writes the new state there directly and leaves the other layers alone."""
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import configs
+    wl = configs.make(1 if version == 5 else 3, B=2, T=128, C=128, H=2, dtype=torch.bfloat16)
+    B, T, C, H = wl.B, wl.T, wl.C, wl.H
+    g = {n: x.cuda() for n, x in wl.tensors.items()}
+    layers = torch.full((3, B, H, 64, 64), 5.0, device="cuda")
+    layers[1].copy_(g["state"])
+    with torch.no_grad():
+        if version == 5:
+            y = W.RUN_WKV5_CUDA(B, T, C, H, layers[1], g["r"], g["k"], g["v"], g["w"], g["u"])
+            y2, s2 = W.WKV_5.apply(B, T, C, H, g["state"], g["r"], g["k"], g["v"], g["w"], g["u"])
+        else:
+            y = W.RUN_WKV6STATE_CUDA(B, T, C, H, g["r"], g["k"], g["v"], g["w"], g["u"], layers[1])
+            y2, s2 = W.WKV_6.apply(B, T, C, H, g["r"], g["k"], g["v"], g["w"], g["u"], g["state"])
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2) and torch.equal(layers[1], s2)
+    assert bool((layers[0] == 5.0).all()) and bool((layers[2] == 5.0).all())
