@@ -51,6 +51,9 @@ def parse():
     ap.add_argument("--w-shift", type=float, default=0.0,
                     help="WKV6 only: added to the raw decay parameter (negative = slower decay; -5 makes every channel "
                          "remember for thousands of tokens, the worst case of the time-parallel split's summary passes)")
+    ap.add_argument("--settle-ms", type=float, default=100.0,
+                    help="untimed replays of the captured steps for this long before the timed region (the first replays "
+                         "of a fresh graph run ~8 %% slower than the steady state a long run measures)")
     ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run three plain 256 MiB device copies first (reference point for the FETCH_SIZE / "
@@ -351,6 +354,11 @@ def main():
             for _ in range(a.steps):
                 runner.step()
 
+    if a.settle_ms > 0 and graph is not None:      # untimed: the first replays of a fresh graph are slower than the steady state
+        t_end = time.perf_counter() + a.settle_ms * 1e-3
+        while time.perf_counter() < t_end:
+            run_k_steps()
+            torch.cuda.synchronize()
     # (1) the K steps between two device synchronisations, by the host's clock.  This includes the latency of the
     # first launch (about 0.2 - 0.6 ms for a graph: the GPU idles until the launch arrives), which is a property
     # of the host, not of the kernels, and weighs 10 % and more on a 20-step run.
@@ -400,7 +408,7 @@ def main():
            "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto",
                       "launch": (f"hip graph of {body_steps} steps per replay" + (f" + one of {a.steps % body_steps}" if tail is not None else ""))
                                 if graph is not None else "eager"},
-           "ms_per_step_host": ms_step_host,
+           "ms_per_step_host": ms_step_host, "untimed_settle_ms": a.settle_ms if graph is not None else 0.0,
            "timing": "ms_per_step and value: HIP events on the launch stream around exactly the K steps, the queue "
                      "primed with two untimed steps; ms_per_step_host: the same K steps between two device "
                      "synchronisations by the host clock (includes the latency of the first launch)",
