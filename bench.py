@@ -48,6 +48,13 @@ def parse():
     ap.add_argument("--w-dtype", default="fp32", choices=["fp32", "bf16"],
                     help="WKV6 only: dtype of the raw decay tensor and its gradient (fp32 is what the workload is "
                          "defined with; bf16 is what a mixed-precision TimeMix hands over)")
+    ap.add_argument("--io-dtype", default="bf16", choices=["bf16", "fp16", "fp32"],
+                    help="WKV5/WKV6: dtype of r, k, v, dy and of y, gr, gk, gv (the workloads are defined in bf16; fp16 and "
+                         "fp32 run the per-token kernels, the reference binds all three, "
+                         "RWKV-v5/src/module/cuda/wkv5_op.cpp:84-129)")
+    ap.add_argument("--helper", action="store_true",
+                    help="time the cumulative-decay helper alone (all tables, chunk length 128) on the raw decay tensor of "
+                         "--cfg 3 instead of the operators")
     ap.add_argument("--w-shift", type=float, default=0.0,
                     help="WKV6 only: added to the raw decay parameter (negative = slower decay; -5 makes every channel "
                          "remember for thousands of tokens, the worst case of the time-parallel split's summary passes)")
@@ -64,7 +71,7 @@ def parse():
 class Runner56:
     """WKV5 / WKV6 forward+backward through the C ABI on preallocated buffers."""
 
-    def __init__(self, cfg, algo, rotate, w_dtype="fp32", w_shift=0.0):
+    def __init__(self, cfg, algo, rotate, w_dtype="fp32", w_shift=0.0, io_dtype="bf16"):
         import torch
         from rwkv_wkv_hip import _lib, configs
         self.torch, self._lib, self.L = torch, _lib, _lib.lib()
@@ -76,6 +83,12 @@ class Runner56:
         self.wl = wl
         self.version = wl.version
         self.w16 = w_dtype == "bf16" and wl.version == 6
+        io = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[io_dtype]
+        if io != wl.dtype:
+            for st in self.sets:
+                for n in ("r", "k", "v", "dy"):
+                    st[n] = st[n].to(io)
+            wl.dtype = io
         if w_shift and wl.version == 6:
             for st in self.sets:
                 st["w"] = st["w"] + w_shift
@@ -105,13 +118,14 @@ class Runner56:
         elems = B * T * C
         st = B * H * 64 * 64 * 4
         wb = 2 if self.w16 else 4                       # bytes of a decay / decay-gradient element
-        fwd_b = (6 + wb + 2) if self.version == 6 else 8
-        bwd_b = (8 + wb + 6 + wb) if self.version == 6 else 14
+        eb = 4 if io == torch.float32 else 2            # bytes of an r, k, v, y, gradient element
+        fwd_b = (4 * eb + wb) if self.version == 6 else 4 * eb
+        bwd_b = (7 * eb + 2 * wb) if self.version == 6 else 7 * eb
         self.bytes_step = (fwd_b + bwd_b) * elems + 5 * st
         self.bytes_fwd = fwd_b * elems + 2 * st
         self.bytes_bwd = bwd_b * elems + 3 * st
-        self.dtype_name = "bf16"
-        self.desc = (f"cfg{cfg}: WKV{self.version} fwd+bwd B{B} T{T} C{C} H{H} head 64, bf16 r/k/v/dy, "
+        self.dtype_name = {"bf16": "bf16", "fp16": "f16", "fp32": "f32"}[io_dtype]
+        self.desc = (f"cfg{cfg}: WKV{self.version} fwd+bwd B{B} T{T} C{C} H{H} head 64, {io_dtype} r/k/v/dy, "
                      f"{'bf16' if self.w16 else 'fp32'} raw decay, fp32 state, state carried step to step, state "
                      f"gradient fed back" + (f", raw decay shifted by {w_shift}" if w_shift else ""))
 
@@ -305,6 +319,41 @@ def measured_traffic(cfg, algo, segments, kernel):
     return rec["traffic_bytes_per_launch"] if same else None
 
 
+def bench_helper(a):
+    """The cumulative-decay helper alone: every table of rwkv_inner.py:43-93 from the raw decay tensor of cfg3
+    (B8 T4096 C2560, chunk length 128).  Algorithmic bytes: 4 read + 4 per fp32 table + 8 per fp64 factor."""
+    import torch
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    wl = configs.make(3)
+    B, T, C = wl.B, wl.T, wl.C
+    w = wl.tensors["w"].cuda().contiguous()
+    f32 = lambda *sh: torch.empty(*sh, dtype=torch.float32, device="cuda")
+    out = [f32(B, T, C) for _ in range(4)] + [f32(B, T // 128, C)]
+    exps = [f32(B, T // 128, C), f32(B, T, C), f32(B, T, C)]
+    facs = [torch.empty(B, T, C, dtype=torch.float64, device="cuda") for _ in range(2)]
+    p = lambda t: t.data_ptr()
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {}
+    for name, fn, nbytes in (
+            ("log_tables", lambda: L.wkv_cumsum_decay(stream, B, T, C, 128, 1, p(w), *[p(t) for t in out]), 20 * B * T * C),
+            ("all_tables", lambda: L.wkv_cumsum_decay_factors(stream, B, T, C, 128, 1, 64, p(w), *[p(t) for t in out + exps + facs]),
+             44 * B * T * C)):
+        for _ in range(max(a.warmup, 3)):
+            assert fn() == 0
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = max(a.steps // 10, 10)
+        ev0.record()
+        for _ in range(n):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        ms = ev0.elapsed_time(ev1) / n
+        res[name] = {"ms": ms, "algorithmic_bytes": nbytes, "GBs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+    print(json.dumps({"metric": "cumulative-decay helper, B8 T4096 C2560, chunk 128", "unit": "ms", "n_gpus": 1, "data": "synthetic",
+                      "dtype": "f32", "value": res["log_tables"]["ms"], "higher_is_better": False, "kernels": res}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -313,7 +362,9 @@ def main():
         sys.exit(2)
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift)
+    if a.helper:
+        return bench_helper(a)
+    runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift, a.io_dtype)
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
     if a.traffic_probe:

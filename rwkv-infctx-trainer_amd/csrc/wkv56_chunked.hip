@@ -43,11 +43,15 @@
 namespace wkv {
 namespace chunked {
 
-// optional per-phase cycle counts of workgroup 0 (development aid, off by default)
+// optional per-phase cycle counts of workgroup 0 (development aid, off by default; build with EXTRA=-DWKV_PHASE_TIMING).
+// forward16:  p5 top of the step, p0 prepare, p1 wait, p2 chains / builders, p3 wait, p4 finish
+// backward16: p5 top of the step (the prefetched inputs arrive), p6 results of the step before written out, p7 running
+//             sum inside the wavefronts + the wait for the others', p0 rest of prepare, p1 wait, p2 chains / builders,
+//             p3 wait, p4 block phase
 #ifdef WKV_PHASE_TIMING
-#define PT_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}; long long pt_last_ = clock64();
+#define PT_DECL long long pt_[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long pt_last_ = clock64();
 #define PT_MARK(i) { const long long now_ = clock64(); pt_[i] += now_ - pt_last_; pt_last_ = now_; }
-#define PT_PRINT(name) if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) printf("%s[%d]: p0 %lld p1 %lld p2 %lld p3 %lld p4 %lld p5 %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5]);
+#define PT_PRINT(name) if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) printf("%s[%d]: p0 %lld p1 %lld p2 %lld p3 %lld p4 %lld p5 %lld p6 %lld p7 %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5], pt_[6], pt_[7]);
 #else
 #define PT_DECL
 #define PT_MARK(i)
@@ -987,7 +991,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                 l[0] = in ? log2_decay(w4.x, floor_decay) : 0.f; l[1] = in ? log2_decay(w4.y, floor_decay) : 0.f;
                 l[2] = in ? log2_decay(w4.z, floor_decay) : 0.f; l[3] = in ? log2_decay(w4.w, floor_decay) : 0.f;
             }
+            PT_MARK(5)
             if (have_out) { write_out(sb + 1, tok, c4, par); par ^= 1; }
+            PT_MARK(6)
             float rhv[4], khv[4], p = 0.f;
             if (whole) {
                 const float4 fr = *reinterpret_cast<const float4 *>(&tab_r[(tok & 15) * HEAD + c4]);
@@ -997,6 +1003,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             } else {
                 scan_local(l, inc, sm.wtot, w16, g, n);      // (the one-step-ahead form of forward16 costs registers this kernel lacks)
                 lds_barrier();
+                PT_MARK(7)
                 scan_join(inc, tot, sm.wtot, w16, n);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
