@@ -192,6 +192,19 @@ __device__ __forceinline__ float row_prefix_sum(float x) {      // inclusive, ov
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));
     return x;
 }
+// inclusive sum over the lanes n..15 of a DPP row (the later tokens of a block when a row's lanes are its 16 tokens)
+__device__ __forceinline__ float row_suffix_sum(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x101, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x102, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x104, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x108, 0xf, 0xf, true));
+    return x;
+}
+// Index into a [token][64 keys] fp32 table of the backward kernel.  The tables are written one token row per 16 lanes
+// (four keys a lane) by the preparing lanes and read one token per lane (four keys) by the block phase; without the
+// exchange of 16-byte pieces inside 128-byte groups by the row number, the second pattern would put eight lanes on
+// the same banks.
+__device__ __forceinline__ int swz(int row, int col) { return row * HEAD + (col ^ ((row & 7) << 2)); }
 // Transposing 8-byte LDS read: with every lane (g, a) of a 16-lane group pointing at
 // tile[row0 + 4g + a/4][col0 + 4(a%4) ..+3], lane (g, n) receives tile[row0 + 4g + i][col0 + n], i = 0..3:
 // an MFMA operand fragment with the rows along the contraction.  `off` = the lane's share of the address.
@@ -816,7 +829,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     const int nsb = (Tlen + SB - 1) / SB;
     const int sb0 = seg * sps, sb1 = min(nsb, (seg + 1) * sps);
     const int own = 16 * wv + n;               // key (or, for the key-major gradient, value) channel of this lane
-    const float u_i = u[h * HEAD + own];
     const float *ck_lane = ckpt + (size_t)bh * (nsb + 1) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
 
     // One register tile set per wavefront, by role:
@@ -868,7 +880,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             if (g == 0) sm.arun[0][own] = a;
         }
     }
-    float gu_acc = 0.f;
+    float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};      // block phase: this lane's token, keys 16wv+4g..+3
+    const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + 16 * wv + 4 * g);      // the bonus of those keys
     float4 gw_acc = make_float4(0.f, 0.f, 0.f, 0.f);      // time-invariant w: sum over this lane's tokens, channels c4..c4+3
 
     // preparing role: token tok of the step (block q), channels c4..c4+3 (one 128-byte row per 16 lanes)
@@ -912,7 +925,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         if (q < 3) { A.x += t3.x; A.y += t3.y; A.z += t3.z; A.w += t3.w; }
         if (q < 2) { A.x += t2.x; A.y += t2.y; A.z += t2.z; A.w += t2.w; }
         if (q < 1) { A.x += t1.x; A.y += t1.y; A.z += t1.z; A.w += t1.w; }
-        const float4 D = *reinterpret_cast<const float4 *>(&sm.incl[tok * HEAD + c4]);
+        const float4 D = *reinterpret_cast<const float4 *>(&sm.incl[swz(tok, c4)]);
         A.x += D.x; A.y += D.y; A.z += D.z; A.w += D.w;
         if (t < Tlen) {
             const size_t o = base + (size_t)t * C + c4;
@@ -920,7 +933,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
             *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
             if (PER_TOKEN_W) {      // dL/dw_raw = dL/dlog w x log w (natural logarithm); nothing where the floor holds
-                const float4 l4 = *reinterpret_cast<const float4 *>(&sm.lw[tok * HEAD + c4]);
+                const float4 l4 = *reinterpret_cast<const float4 *>(&sm.lw[swz(tok, c4)]);
                 const float lf[4] = {l4.x, l4.y, l4.z, l4.w};
                 float f[4];
 #pragma unroll
@@ -952,8 +965,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
       if (whole && !tables_valid) {
           const int key = tid & 63, pl = tid >> 6;
           const float lk = log2_decay(static_cast<const float *>(wraw)[h * HEAD + key], floor_decay);
-          tab_r[pl * HEAD + key] = exp2_fast(pl * lk);
-          tab_k[pl * HEAD + key] = exp2_fast((15 - pl) * lk);
+          tab_r[swz(pl, key)] = exp2_fast(pl * lk);
+          tab_k[swz(pl, key)] = exp2_fast((15 - pl) * lk);
           if (pl < 4) {
               sm.tot[pl][key] = 16.f * lk;
               sm.dec[pl][key] = exp2_fast(16.f * lk);
@@ -996,8 +1009,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             PT_MARK(6)
             float rhv[4], khv[4], p = 0.f;
             if (whole) {
-                const float4 fr = *reinterpret_cast<const float4 *>(&tab_r[(tok & 15) * HEAD + c4]);
-                const float4 fk = *reinterpret_cast<const float4 *>(&tab_k[(tok & 15) * HEAD + c4]);
+                const float4 fr = *reinterpret_cast<const float4 *>(&tab_r[swz(tok & 15, c4)]);
+                const float4 fk = *reinterpret_cast<const float4 *>(&tab_k[swz(tok & 15, c4)]);
                 rhv[0] = rf[0] * fr.x; rhv[1] = rf[1] * fr.y; rhv[2] = rf[2] * fr.z; rhv[3] = rf[3] * fr.w;
                 khv[0] = kf[0] * fk.x; khv[1] = kf[1] * fk.y; khv[2] = kf[2] * fk.z; khv[3] = kf[3] * fk.w;
             } else {
@@ -1023,12 +1036,12 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             split2(khv[0], khv[1], h0, l0); split2(khv[2], khv[3], h1, l1);
             *reinterpret_cast<uint2 *>(&sm.kh[o]) = make_uint2(h0, h1);
             *reinterpret_cast<uint2 *>(&sm.khl[o]) = make_uint2(l0, l1);
-            *reinterpret_cast<uint4 *>(&sm.rk[tok * HEAD + c4]) =
+            *reinterpret_cast<uint4 *>(&sm.rk[swz(tok, c4)]) =
                 make_uint4((pr.x & 0xffffu) | (pk.x << 16), (pr.x >> 16) | (pk.x & 0xffff0000u),
                            (pr.y & 0xffffu) | (pk.y << 16), (pr.y >> 16) | (pk.y & 0xffff0000u));
             if (!whole) {
-                *reinterpret_cast<float4 *>(&sm.incl[tok * HEAD + c4]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
-                *reinterpret_cast<float4 *>(&sm.lw[tok * HEAD + c4]) = make_float4(l[0], l[1], l[2], l[3]);
+                *reinterpret_cast<float4 *>(&sm.incl[swz(tok, c4)]) = make_float4(inc[0], inc[1], inc[2], inc[3]);
+                *reinterpret_cast<float4 *>(&sm.lw[swz(tok, c4)]) = make_float4(l[0], l[1], l[2], l[3]);
             }
             if (!whole && (w16 & 3) == 3) {       // wavefront-uniform: only the wavefront with the block's last token
                 if (g == 3) {
@@ -1059,11 +1072,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                     split4(G[kk], s0h, s0l);
                     split4(G[kk + 1], s1h, s1l);
                     const s4 y0 = frag(sm.gy, 16 * qq + n, 16 * kk + 4 * g), y1 = frag(sm.gy, 16 * qq + n, 16 * kk + 16 + 4 * g);
-                    qa = mma2(y0, y1, s0l, s1l, qa);
-                    qa = mma2(y0, y1, s0h, s1h, qa);
+                    qa = mma2(s0l, s1l, y0, y1, qa);       // (the state as the A operand: the product comes out as [key][token])
+                    qa = mma2(s0h, s1h, y0, y1, qa);
                 }
-#pragma unroll
-                for (int e = 0; e < 4; e++) sm.q1[(16 * qq + 4 * g + e) * HEAD + own] = qa[e];
+                *reinterpret_cast<float4 *>(&sm.q1[swz(16 * qq + n, 16 * wv + 4 * g)]) = make_float4(qa[0], qa[1], qa[2], qa[3]);
                 if (qq < 3) {
                     const float dq = sm.dec[qq][own];
                     const s4 khf = frag_tr(sm.kh, tro + (16 * qq) * LD + 16 * wv), khfl = frag_tr(sm.khl, tro + (16 * qq) * LD + 16 * wv);
@@ -1086,11 +1098,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                     split4(G[kk], g0h, g0l);
                     split4(G[kk + 1], g1h, g1l);
                     const s4 v0 = frag(sm.v, 16 * qq + n, 16 * kk + 4 * g), v1 = frag(sm.v, 16 * qq + n, 16 * kk + 16 + 4 * g);
-                    q4 = mma2(v0, v1, g0l, g1l, q4);
-                    q4 = mma2(v0, v1, g0h, g1h, q4);
+                    q4 = mma2(g0l, g1l, v0, v1, q4);
+                    q4 = mma2(g0h, g1h, v0, v1, q4);
                 }
-#pragma unroll
-                for (int e = 0; e < 4; e++) sm.q4[(16 * qq + 4 * g + e) * HEAD + own] = q4[e];
+                *reinterpret_cast<float4 *>(&sm.q4[swz(16 * qq + n, 16 * wv + 4 * g)]) = make_float4(q4[0], q4[1], q4[2], q4[3]);
                 const float dq = sm.dec[qq][own];
                 const s4 rhTf = frag_tr(sm.rh, tro + (16 * qq) * LD + 16 * wv), rhTfl = frag_tr(sm.rhl, tro + (16 * qq) * LD + 16 * wv);
 #pragma unroll
@@ -1113,9 +1124,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                     split4(G[kk], g0h, g0l);
                     split4(G[kk + 1], g1h, g1l);
                     const s4 h0 = frag(sm.kh, row, ca), h1 = frag(sm.kh, row, cb);
-                    g0 = mma2(h0, h1, g0l, g1l, g0);
-                    g0 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0h, g1h, g0);
-                    g0 = mma2(h0, h1, g0h, g1h, g0);
+                    g0 = mma2(g0l, g1l, h0, h1, g0);       // (the gradient as the A operand: [value][token])
+                    g0 = mma2(g0h, g1h, frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0);
+                    g0 = mma2(g0h, g1h, h0, h1, g0);
                 }
                 KG[qq] = g0;
                 if (qq == 3) sm.kg3[wv][lane] = make_float4(KG[3][0], KG[3][1], KG[3][2], KG[3][3]);
@@ -1192,68 +1203,76 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 
       {
         WKV_LOCAL_LANE
+        // In this phase the products come out transposed, [channel][token]: a lane holds four consecutive channels
+        // of one token (token 16 blk + n, channels 16 wv + 4 g ..), so every table access is one 16-byte piece, the
+        // results go into their tiles eight bytes at a time, and the sums over a block's tokens run along a DPP row.
         if (role == 2) {
-            // ---------------- gv[s][value own] = kh G + sum_{t>=s} A~[t][s] gy[t]
+            // ---------------- gv[s][value] = kh G + sum_{t>=s} A~[t][s] gy[t], values 16wv..16wv+15
 #pragma unroll
             for (int qq = 0; qq < 4; qq++) {
                 const uint4 am = sm.amat[qq][lane];
                 const s4 gyTf = frag_tr(sm.gy, tro + (16 * qq) * LD + 16 * wv);
                 f4 kgq = KG[qq < 3 ? qq : 0];
                 if (qq == 3) { const float4 t4 = sm.kg3[wv][lane]; kgq = f4{t4.x, t4.y, t4.z, t4.w}; }
-                const f4 gvt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), gyTf, gyTf, kgq);
-#pragma unroll
-                for (int e = 0; e < 4; e++) sm.v[(16 * qq + 4 * g + e) * LD + own] = bf16_bits(gvt[e]);      // v is not read any more
+                const f4 gvt = mma2(gyTf, gyTf, as_s4(am.x, am.y), as_s4(am.z, am.w), kgq);
+                *reinterpret_cast<uint2 *>(&sm.v[(16 * qq + n) * LD + 16 * wv + 4 * g]) =
+                    make_uint2(bf16_pack2(gvt[0], gvt[1]), bf16_pack2(gvt[2], gvt[3]));      // v is not read any more
             }
         }
-        // ---------------- block q, keys 16wv..16wv+15: gr, gk, decay gradient
+        // ---------------- block q, token 16q+n, keys 16wv+4g..+3: gr, gk, decay gradient
         {
             const uint4 pa = sm.pfr[q][0][lane], pb = sm.pfr[q][1][lane];
             const s4 pT_h = as_s4(pa.x, pa.y), pT_l = as_s4(pa.z, pa.w), pm_h = as_s4(pb.x, pb.y), pm_l = as_s4(pb.z, pb.w);
             const s4 khTf = frag_tr(sm.kh, tro + (16 * q) * LD + 16 * wv), khTfl = frag_tr(sm.khl, tro + (16 * q) * LD + 16 * wv);
             const s4 rhTf = frag_tr(sm.rh, tro + (16 * q) * LD + 16 * wv), rhTfl = frag_tr(sm.rhl, tro + (16 * q) * LD + 16 * wv);
             f4 q2 = {0.f, 0.f, 0.f, 0.f}, q3 = q2;
-            q2 = mma(pT_h, khTfl, q2);
-            q3 = mma(pm_h, rhTfl, q3);
-            q2 = mma2(pT_h, pT_l, khTf, khTf, q2);      // sum_{s<t} P[t][s] kh_s
-            q3 = mma2(pm_h, pm_l, rhTf, rhTf, q3);      // sum_{t>s} P[t][s] rh_t
-            const float tot_i = sm.tot[q][own], ent_i = sm.ent[q][own];
-            float c[4], z[4];
+            q2 = mma(khTfl, pT_h, q2);
+            q3 = mma(rhTfl, pm_h, q3);
+            q2 = mma2(khTf, khTf, pT_h, pT_l, q2);      // sum_{s<t} P[t][s] kh_s   at [key][t]
+            q3 = mma2(rhTf, rhTf, pm_h, pm_l, q3);      // sum_{t>s} P[t][s] rh_t   at [key][s]
+            const int tk = 16 * q + n, k4 = 16 * wv + 4 * g, ti = swz(tk, k4);
+            const float4 tot4 = *reinterpret_cast<const float4 *>(&sm.tot[q][k4]), ent4 = *reinterpret_cast<const float4 *>(&sm.ent[q][k4]);
+            const float4 q1v = *reinterpret_cast<const float4 *>(&sm.q1[ti]), q4v = *reinterpret_cast<const float4 *>(&sm.q4[ti]);
+            const uint4 rk4 = *reinterpret_cast<const uint4 *>(&sm.rk[ti]);
+            const float pd = sm.pdiag[q][n];
+            float E1[4], E2[4];
+            if (whole) {
+                const float4 fr = *reinterpret_cast<const float4 *>(&tab_r[swz(n, k4)]), fk = *reinterpret_cast<const float4 *>(&tab_k[swz(n, k4)]);
+                E1[0] = fr.x; E1[1] = fr.y; E1[2] = fr.z; E1[3] = fr.w;
+                E2[0] = fk.x; E2[1] = fk.y; E2[2] = fk.z; E2[3] = fk.w;
+            } else {
+                const float4 in4 = *reinterpret_cast<const float4 *>(&sm.incl[ti]), lw4 = *reinterpret_cast<const float4 *>(&sm.lw[ti]);
+                E1[0] = exp2_fast(in4.x - lw4.x); E1[1] = exp2_fast(in4.y - lw4.y); E1[2] = exp2_fast(in4.z - lw4.z); E1[3] = exp2_fast(in4.w - lw4.w);
+                E2[0] = exp2_fast(tot4.x - in4.x); E2[1] = exp2_fast(tot4.y - in4.y); E2[2] = exp2_fast(tot4.z - in4.z); E2[3] = exp2_fast(tot4.w - in4.w);
+            }
+            const float entf[4] = {ent4.x, ent4.y, ent4.z, ent4.w}, uf[4] = {u4.x, u4.y, u4.z, u4.w};
+            const float q1f[4] = {q1v.x, q1v.y, q1v.z, q1v.w}, q4f[4] = {q4v.x, q4v.y, q4v.z, q4v.w};
+            const uint32_t rkf[4] = {rk4.x, rk4.y, rk4.z, rk4.w};
+            float c[4], z[4], grv[4], gkv[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int tk = 16 * q + 4 * g + e;
-                float E1, E2;
-                if (whole) {
-                    E1 = tab_r[(4 * g + e) * HEAD + own];
-                    E2 = tab_k[(4 * g + e) * HEAD + own];
-                } else {
-                    const float inc = sm.incl[tk * HEAD + own];
-                    E1 = exp2_fast(inc - sm.lw[tk * HEAD + own]);
-                    E2 = exp2_fast(tot_i - inc);
-                }
-                const float q1 = sm.q1[tk * HEAD + own], q4 = sm.q4[tk * HEAD + own], pd = sm.pdiag[q][4 * g + e];
-                const uint32_t rkv = sm.rk[tk * HEAD + own];
-                const float rr = bf_lo(rkv), kr = bf_hi(rkv);
-                const float grv = E1 * (q1 + ent_i * q2[e]) + u_i * kr * pd;
-                const float gkn = E2 * (ent_i * q3[e] + q4);
-                const float gkv = gkn + u_i * rr * pd;
-                c[e] = rr * grv - kr * gkv;
+                const float rr = bf_lo(rkf[e]), kr = bf_hi(rkf[e]), upd = uf[e] * pd;
+                grv[e] = E1[e] * (q1f[e] + entf[e] * q2[e]) + upd * kr;
+                const float gkn = E2[e] * (entf[e] * q3[e] + q4f[e]);
+                gkv[e] = gkn + upd * rr;
+                c[e] = rr * grv[e] - kr * gkv[e];
                 z[e] = kr * gkn;
-                gu_acc = fmaf(rr * kr, pd, gu_acc);
-                // this wavefront was the only reader left of its (block, quarter) corner of the rh and kh tiles
-                sm.rh[tk * LD + own] = bf16_bits(grv);
-                sm.kh[tk * LD + own] = bf16_bits(gkv);
+                gu_acc[e] = fmaf(rr * kr, pd, gu_acc[e]);
             }
+            // this wavefront was the only reader left of its (block, quarter) corner of the rh and kh tiles
+            *reinterpret_cast<uint2 *>(&sm.rh[tk * LD + k4]) = make_uint2(bf16_pack2(grv[0], grv[1]), bf16_pack2(grv[2], grv[3]));
+            *reinterpret_cast<uint2 *>(&sm.kh[tk * LD + k4]) = make_uint2(bf16_pack2(gkv[0], gkv[1]), bf16_pack2(gkv[2], gkv[3]));
             // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over the block's later tokens of c
-            const float suf2 = c[3], suf1 = c[3] + c[2], suf0 = suf1 + c[1], mine = suf0 + c[0];
-            const float t1 = __shfl_down(mine, 16), t2 = __shfl_down(mine, 32), t3 = __shfl_down(mine, 48);
-            const float later = (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);
-            const float all = group_sum4(mine);
+            float dpart[4], all[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float incl_suf = row_suffix_sum(c[e]);          // c of this token and the later ones
+                dpart[e] = (incl_suf - c[e]) - z[e];
+                all[e] = incl_suf;                                    // (lane n = 0: the whole block)
+            }
             // (the incl entries of this block and quarter had this wavefront as their only reader)
-            sm.incl[(16 * q + 4 * g + 0) * HEAD + own] = later + suf0 - z[0];
-            sm.incl[(16 * q + 4 * g + 1) * HEAD + own] = later + suf1 - z[1];
-            sm.incl[(16 * q + 4 * g + 2) * HEAD + own] = later + suf2 - z[2];
-            sm.incl[(16 * q + 4 * g + 3) * HEAD + own] = later - z[3];
-            if (g == 0) sm.tots[q][own] = all;
+            *reinterpret_cast<float4 *>(&sm.incl[ti]) = make_float4(dpart[0], dpart[1], dpart[2], dpart[3]);
+            if (n == 0) *reinterpret_cast<float4 *>(&sm.tots[q][k4]) = make_float4(all[0], all[1], all[2], all[3]);
         }
       }
         PT_MARK(4)
@@ -1269,8 +1288,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         for (int kk = 0; kk < 4; kk++)
             *reinterpret_cast<float4 *>(gp + 16 * kk + 4 * g) = make_float4(G[kk][0], G[kk][1], G[kk][2], G[kk][3]);
     }
-    gu_acc = group_sum4(gu_acc);
-    if (g == 0) sm.red[q][own] = gu_acc;
+#pragma unroll
+    for (int e = 0; e < 4; e++) gu_acc[e] = row_suffix_sum(gu_acc[e]);       // lane n = 0: the sum over the row's 16 tokens
+    if (n == 0) *reinterpret_cast<float4 *>(&sm.red[q][16 * wv + 4 * g]) = make_float4(gu_acc[0], gu_acc[1], gu_acc[2], gu_acc[3]);
     float *gw16 = sm.q1;            // [16][HEAD]; the q1 table is dead by now
     if (!PER_TOKEN_W) {
         gw_acc.x = group_sum4(gw_acc.x); gw_acc.y = group_sum4(gw_acc.y);
