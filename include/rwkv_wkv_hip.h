@@ -207,6 +207,55 @@ int wkv_cumsum_decay_factors(void *stream, int Bw, int T, int C, int chunk_len, 
                              const float *w, float *log_w, float *incl, float *inter, float *intra, float *chunk_sum,
                              float *ws_exp, float *inter_exp, float *intra_exp, void *r_decay, void *k_inv_decay);
 
+/* ---- The element-wise passes on either side of the operator inside a block.  Tensors are contiguous (.., C)
+ * in `dtype`; parameters (coef, weight, bias) and their gradients are fp32.  None of these allocates. */
+
+/* Token shift + mixing (RWKV-v5/src/module/TimeMix.py:292-298 and ChannelMix.py:44-47 with lerp = 1;
+ * RWKV-v6/src/module/TimeMix.py:262-276 and ChannelMix.py:31-35 with lerp = 0): from one read of x,
+ *   out[j][b,t,:] = x[b,t,:] + (x[b,t-1,:] - x[b,t,:]) * d_j,   x[b,-1,:] = shift[b,:]
+ * for j < n (n <= 5).  lerp = 1: coef[j] is the reference's time_mix_j, d_j = 1 - coef[j] (modified_lerp,
+ * RWKV-v5/src/module/OptimizedOps.py:14-15).  lerp = 0: coef[j] is time_maa_j, d_j = coef[j] + dyn[j][b,t,:], with
+ * dyn (n, B, T, C) the data-dependent part (the reference's mw, mk, mv, mr, mg, RWKV-v6 TimeMix.py:265-268) or NULL.
+ *   x (B,T,C); shift (B,C); coef (n,C) fp32; out: HOST array of n device pointers, each (B,T,C). */
+int wkv_shift_mix_forward(void *stream, int B, int T, int C, int dtype, int n, int lerp, const void *x,
+                          const void *shift, const float *coef, const void *dyn, void *const *out);
+
+/* Its backward (what autograd derives from the lines cited above): gout = HOST array of the n output gradients;
+ * gx (B,T,C), gshift (B,C) in `dtype`; gcoef (n,C) fp32, summed over batch and time in a fixed order; gdyn
+ * (n,B,T,C) in `dtype`, required when dyn is given.  workspace: wkv_shift_mix_backward_workspace bytes. */
+size_t wkv_shift_mix_backward_workspace(int B, int T, int C, int n);
+int wkv_shift_mix_backward(void *stream, int B, int T, int C, int dtype, int n, int lerp, const void *x,
+                           const void *shift, const float *coef, const void *dyn, const void *const *gout, void *gx,
+                           void *gshift, float *gcoef, void *gdyn, void *workspace, size_t workspace_bytes);
+
+/* ln_x and the gate on the operator's output (RWKV-v5/src/module/TimeMix.py:301,317-320: scale = 1/8, eps = 1e-5;
+ * RWKV-v6/src/module/TimeMix.py:180,278,296-298: scale = 1, eps = 64e-5):
+ *   out = (GroupNorm(y * scale; one group per 64-channel head, eps) * weight + bias) * silu(gate)
+ * gate is the gate projection BEFORE its SiLU (the reference applies F.silu first and multiplies afterwards; here
+ * both happen in the one pass), or NULL for the normalisation alone.  rows = B*T; y, gate, out (rows, C). */
+int wkv_ln_gate_forward(void *stream, int rows, int C, int dtype, float scale, float eps, const void *y,
+                        const void *gate, const float *weight, const float *bias, void *out);
+
+/* Its backward: gy, ggate (w.r.t. the gate projection) in `dtype`; gweight_gbias (2, C) fp32 = gradient of weight,
+ * then of bias, summed over rows in a fixed order.  workspace: wkv_ln_gate_backward_workspace bytes. */
+size_t wkv_ln_gate_backward_workspace(int rows, int C);
+int wkv_ln_gate_backward(void *stream, int rows, int C, int dtype, float scale, float eps, const void *y,
+                         const void *gate, const float *weight, const float *bias, const void *gout, void *gy,
+                         void *ggate, float *gweight_gbias, void *workspace, size_t workspace_bytes);
+
+/* The activations of the channel mix (RWKV-v5/src/module/ChannelMix.py:48-49, RWKV-v6/src/module/ChannelMix.py:
+ * 36-37) over n elements (n a multiple of 8): out = relu(k)^2;  out = sigmoid(r) * kv; and their backwards. */
+int wkv_relu_square_forward(void *stream, size_t n, int dtype, const void *k, void *out);
+int wkv_relu_square_backward(void *stream, size_t n, int dtype, const void *k, const void *gout, void *gk);
+int wkv_sigmoid_mul_forward(void *stream, size_t n, int dtype, const void *r, const void *kv, void *out);
+int wkv_sigmoid_mul_backward(void *stream, size_t n, int dtype, const void *r, const void *kv, const void *gout,
+                             void *gr, void *gkv);
+
+/* Backward of L2Wrap (RWKV-v5/src/model.py:140-148): gy (rows, V) is zero except, in every row, at the first
+ * position of the row's maximum, where it is factor * mask[row] * max (mask (rows) fp32 or NULL = ones). */
+int wkv_l2wrap_backward(void *stream, int rows, int V, int dtype, float factor, const void *y, const float *mask,
+                        void *gy);
+
 #ifdef __cplusplus
 }
 #endif

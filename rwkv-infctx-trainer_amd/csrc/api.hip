@@ -8,6 +8,7 @@
 #include "wkv56_noalloc.hip"
 #include "wkv4.hip"
 #include "cumsum_decay.hip"
+#include "block_edges.hip"
 
 using namespace wkv;
 
@@ -294,6 +295,147 @@ int wkv_cumsum_decay_factors(void *stream, int Bw, int T, int C, int chunk_len, 
     if (!w) return WKV_ERR_NULL;
     hipError_t e = cumsum_decay_factors_launch((hipStream_t)stream, Bw, T, C, chunk_len, per_token, precision, w, log_w, incl,
                                                inter, intra, chunk_sum, ws_exp, inter_exp, intra_exp, r_decay, k_inv_decay);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+// ---- the element-wise passes around the operator (block_edges.hip)
+#define WKV_BY_DTYPE(dtype, CALL)                                   \
+    ((dtype) == WKV_BF16 ? CALL(bf16) : (dtype) == WKV_F16 ? CALL(f16) : CALL(float))
+
+size_t wkv_shift_mix_backward_workspace(int B, int T, int C, int n) {
+    if (B <= 0 || T <= 0 || C <= 0 || n <= 0 || n > edges::MAX_MIX) return 0;
+    return edges::shift_mix_backward_workspace(B, T, C, n);
+}
+
+int wkv_shift_mix_forward(void *stream, int B, int T, int C, int dtype, int n, int lerp, const void *x, const void *shift,
+                          const float *coef, const void *dyn, void *const *out) {
+    if (B <= 0 || T <= 0 || C <= 0 || C % 8 != 0 || B > 65535 || n <= 0 || n > edges::MAX_MIX) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    if (!x || !shift || !coef || !out) return WKV_ERR_NULL;
+    for (int j = 0; j < n; j++) {
+        if (!out[j]) return WKV_ERR_NULL;
+        if (!aligned16(out[j])) return WKV_ERR_ALIGN;
+    }
+    for (const void *p : {x, shift, (const void *)coef, dyn})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::shift_mix_forward_t<TY>((hipStream_t)stream, B, T, C, n, lerp, x, shift, coef, dyn, out)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_shift_mix_backward(void *stream, int B, int T, int C, int dtype, int n, int lerp, const void *x, const void *shift,
+                           const float *coef, const void *dyn, const void *const *gout, void *gx, void *gshift, float *gcoef,
+                           void *gdyn, void *workspace, size_t workspace_bytes) {
+    if (B <= 0 || T <= 0 || C <= 0 || C % 8 != 0 || B > 65535 || n <= 0 || n > edges::MAX_MIX) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    if (!x || !shift || !coef || !gout || !gx || !gshift || !gcoef || !workspace || (dyn && !gdyn)) return WKV_ERR_NULL;
+    for (int j = 0; j < n; j++) {
+        if (!gout[j]) return WKV_ERR_NULL;
+        if (!aligned16(gout[j])) return WKV_ERR_ALIGN;
+    }
+    for (const void *p : {x, shift, (const void *)coef, dyn, (const void *)gx, (const void *)gshift, (const void *)gcoef,
+                          (const void *)gdyn, (const void *)workspace})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    if (workspace_bytes < edges::shift_mix_backward_workspace(B, T, C, n)) return WKV_ERR_WORKSPACE;
+#define CALL(TY) edges::shift_mix_backward_t<TY>((hipStream_t)stream, B, T, C, n, lerp, x, shift, coef, dyn, gout, gx, gshift, \
+                                                 gcoef, gdyn, (float *)workspace)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+size_t wkv_ln_gate_backward_workspace(int rows, int C) {
+    if (rows <= 0 || C <= 0) return 0;
+    return edges::ln_gate_backward_workspace(rows, C);
+}
+
+int wkv_ln_gate_forward(void *stream, int rows, int C, int dtype, float scale, float eps, const void *y, const void *gate,
+                        const float *weight, const float *bias, void *out) {
+    if (rows <= 0 || C <= 0 || C % HEAD != 0 || (rows + edges::TILE_R - 1) / edges::TILE_R > 65535) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    if (!y || !weight || !bias || !out) return WKV_ERR_NULL;
+    for (const void *p : {y, gate, (const void *)weight, (const void *)bias, (const void *)out})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::ln_gate_forward_t<TY>((hipStream_t)stream, rows, C, scale, eps, y, gate, weight, bias, out)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_ln_gate_backward(void *stream, int rows, int C, int dtype, float scale, float eps, const void *y, const void *gate,
+                         const float *weight, const float *bias, const void *gout, void *gy, void *ggate,
+                         float *gweight_gbias, void *workspace, size_t workspace_bytes) {
+    if (rows <= 0 || C <= 0 || C % HEAD != 0 || (rows + edges::TILE_R - 1) / edges::TILE_R > 65535) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    if (!y || !weight || !bias || !gout || !gy || !gweight_gbias || !workspace || (gate && !ggate)) return WKV_ERR_NULL;
+    for (const void *p : {y, gate, (const void *)weight, (const void *)bias, gout, (const void *)gy, (const void *)ggate,
+                          (const void *)gweight_gbias, (const void *)workspace})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    if (workspace_bytes < edges::ln_gate_backward_workspace(rows, C)) return WKV_ERR_WORKSPACE;
+#define CALL(TY) edges::ln_gate_backward_t<TY>((hipStream_t)stream, rows, C, scale, eps, y, gate, weight, bias, gout, gy, ggate, \
+                                               gweight_gbias, (float *)workspace)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+static int check_flat(size_t n, int dtype) {
+    if (n == 0 || n % 8 != 0 || n / 8 / 256 >= (1u << 31)) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    return WKV_OK;
+}
+
+int wkv_relu_square_forward(void *stream, size_t n, int dtype, const void *k, void *out) {
+    if (int st = check_flat(n, dtype)) return st;
+    if (!k || !out) return WKV_ERR_NULL;
+    if (!aligned16(k) || !aligned16(out)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::relu_square_forward_t<TY>((hipStream_t)stream, n, k, out)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_relu_square_backward(void *stream, size_t n, int dtype, const void *k, const void *gout, void *gk) {
+    if (int st = check_flat(n, dtype)) return st;
+    if (!k || !gout || !gk) return WKV_ERR_NULL;
+    if (!aligned16(k) || !aligned16(gout) || !aligned16(gk)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::relu_square_backward_t<TY>((hipStream_t)stream, n, k, gout, gk)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_sigmoid_mul_forward(void *stream, size_t n, int dtype, const void *r, const void *kv, void *out) {
+    if (int st = check_flat(n, dtype)) return st;
+    if (!r || !kv || !out) return WKV_ERR_NULL;
+    if (!aligned16(r) || !aligned16(kv) || !aligned16(out)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::sigmoid_mul_forward_t<TY>((hipStream_t)stream, n, r, kv, out)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_sigmoid_mul_backward(void *stream, size_t n, int dtype, const void *r, const void *kv, const void *gout, void *gr,
+                             void *gkv) {
+    if (int st = check_flat(n, dtype)) return st;
+    if (!r || !kv || !gout || !gr || !gkv) return WKV_ERR_NULL;
+    for (const void *p : {r, kv, gout, (const void *)gr, (const void *)gkv})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::sigmoid_mul_backward_t<TY>((hipStream_t)stream, n, r, kv, gout, gr, gkv)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_l2wrap_backward(void *stream, int rows, int V, int dtype, float factor, const void *y, const float *mask, void *gy) {
+    if (rows <= 0 || V <= 0) return WKV_ERR_DIMS;
+    if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
+    if (!y || !gy) return WKV_ERR_NULL;
+    if (!aligned16(y) || !aligned16(gy)) return WKV_ERR_ALIGN;
+#define CALL(TY) edges::l2wrap_backward_t<TY>((hipStream_t)stream, rows, V, factor, y, mask, gy)
+    hipError_t e = WKV_BY_DTYPE(dtype, CALL);
+#undef CALL
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
 

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_size_t, c_uint, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_uint, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RWKV_WKV_LIB", os.path.join(_HERE, "librwkv_wkv_hip.so"))
@@ -45,6 +45,17 @@ SIGNATURES = {
     "wkv4_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, c_size_t]),
     "wkv_cumsum_decay": (_I, [_P, _I, _I, _I, _I, _I] + [_P] * 6),
     "wkv_cumsum_decay_factors": (_I, [_P, _I, _I, _I, _I, _I, _I] + [_P] * 11),
+    "wkv_shift_mix_forward": (_I, [_P, _I, _I, _I, _I, _I, _I] + [_P] * 5),
+    "wkv_shift_mix_backward_workspace": (c_size_t, [_I] * 4),
+    "wkv_shift_mix_backward": (_I, [_P, _I, _I, _I, _I, _I, _I] + [_P] * 9 + [_P, c_size_t]),
+    "wkv_ln_gate_forward": (_I, [_P, _I, _I, _I, c_float, c_float] + [_P] * 5),
+    "wkv_ln_gate_backward_workspace": (c_size_t, [_I] * 2),
+    "wkv_ln_gate_backward": (_I, [_P, _I, _I, _I, c_float, c_float] + [_P] * 8 + [_P, c_size_t]),
+    "wkv_relu_square_forward": (_I, [_P, c_size_t, _I, _P, _P]),
+    "wkv_relu_square_backward": (_I, [_P, c_size_t, _I, _P, _P, _P]),
+    "wkv_sigmoid_mul_forward": (_I, [_P, c_size_t, _I, _P, _P, _P]),
+    "wkv_sigmoid_mul_backward": (_I, [_P, c_size_t, _I] + [_P] * 5),
+    "wkv_l2wrap_backward": (_I, [_P, _I, _I, _I, c_float, _P, _P, _P]),
 }
 
 _lib = None

@@ -66,6 +66,22 @@ def test_argument_checks_return_before_any_launch(L):
     assert L.wkv4_forward(null, 0, 8, 64, 0, one, one, one, one, null, one, null, null) == -1
     assert L.wkv4_backward(null, 1, 8, 64, 0, *([one] * 13), one, 0) == -5
     assert L.wkv_cumsum_decay(null, 1, 100, 64, 16, 1, one, null, null, null, null, null) == -1
+    # the element-wise passes around the operator
+    outs = (ctypes.c_void_p * 2)(16, 16)
+    assert L.wkv_shift_mix_forward(null, 1, 8, 100, 1, 2, 1, one, one, one, null, outs) == -1        # C % 8
+    assert L.wkv_shift_mix_forward(null, 1, 8, 64, 1, 6, 1, one, one, one, null, outs) == -1         # more than 5 mixes
+    assert L.wkv_shift_mix_forward(null, 1, 8, 64, 1, 2, 1, one, null, one, null, outs) == -2
+    assert L.wkv_shift_mix_forward(null, 1, 8, 64, 1, 2, 1, one, one, one, null, (ctypes.c_void_p * 2)(16, 24)) == -4
+    need = L.wkv_shift_mix_backward_workspace(1, 8, 64, 2)
+    assert need == 1 * 1 * 2 * 64 * 4
+    assert L.wkv_shift_mix_backward(null, 1, 8, 64, 1, 2, 1, one, one, one, null, outs, one, one, one, null, one, need - 1) == -5
+    assert L.wkv_shift_mix_backward(null, 1, 8, 64, 1, 2, 0, one, one, one, one, outs, one, one, one, null, one, need) == -2  # dyn, no gdyn
+    assert L.wkv_ln_gate_forward(null, 4, 96, 1, 1.0, 1e-5, one, one, one, one, one) == -1           # C % 64
+    assert L.wkv_ln_gate_backward(null, 4, 64, 1, 1.0, 1e-5, one, one, one, one, one, one, null, one, one, 1 << 20) == -2
+    assert L.wkv_ln_gate_backward(null, 4, 64, 1, 1.0, 1e-5, one, one, one, one, one, one, one, one, one, 8) == -5
+    assert L.wkv_relu_square_forward(null, 12, 1, one, one) == -1                                    # n % 8
+    assert L.wkv_sigmoid_mul_backward(null, 16, 9, one, one, one, one, one) == -3
+    assert L.wkv_l2wrap_backward(null, 0, 8, 1, 1.0, one, null, one) == -1
 
 
 def test_python_front_end_rejects_cpu_tensors():

@@ -93,3 +93,41 @@ class TimeMix6(nn.Module):
         y, new_state = wkv(B, T, C, H, r, k, v, w.contiguous(), self.time_faaaa, last_state[1])
         y = group_norm(self.ln_x, y.reshape(-1, C), H).view(B, T, C)
         return self.output(y * gate), (x[:, -1], new_state)
+
+
+class ChannelMix5(nn.Module):
+    """RWKV-v5/src/module/ChannelMix.py:7-49 with seeded parameters; forward = the oracle's restatement"""
+    def __init__(self, n_embd, dim_ffn, seed=0):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.time_mix_k = nn.Parameter(torch.rand(1, 1, n_embd, generator=g))
+        self.time_mix_r = nn.Parameter(torch.rand(1, 1, n_embd, generator=g))
+        self.key = nn.Linear(n_embd, dim_ffn, bias=False)
+        self.receptance = nn.Linear(n_embd, n_embd, bias=False)
+        self.value = nn.Linear(dim_ffn, n_embd, bias=False)
+        with torch.no_grad():
+            for m in (self.key, self.receptance, self.value):
+                m.weight.copy_(torch.randn(m.weight.shape, generator=g) * (m.weight.shape[1] ** -0.5))
+
+    def forward(self, x, last_state):
+        from oracle.blocks import channelmix5_forward
+        return channelmix5_forward(self, x, last_state)
+
+
+class ChannelMix6(nn.Module):
+    """RWKV-v6/src/module/ChannelMix.py:7-37 with seeded parameters"""
+    def __init__(self, n_embd, dim_ffn, seed=0):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.time_maa_k = nn.Parameter(torch.rand(1, 1, n_embd, generator=g))
+        self.time_maa_r = nn.Parameter(torch.rand(1, 1, n_embd, generator=g))
+        self.key = nn.Linear(n_embd, dim_ffn, bias=False)
+        self.receptance = nn.Linear(n_embd, n_embd, bias=False)
+        self.value = nn.Linear(dim_ffn, n_embd, bias=False)
+        with torch.no_grad():
+            for m in (self.key, self.receptance, self.value):
+                m.weight.copy_(torch.randn(m.weight.shape, generator=g) * (m.weight.shape[1] ** -0.5))
+
+    def forward(self, x, last_state):
+        from oracle.blocks import channelmix6_forward
+        return channelmix6_forward(self, x, last_state)
