@@ -55,6 +55,9 @@ def parse():
     ap.add_argument("--helper", action="store_true",
                     help="time the cumulative-decay helper alone (all tables, chunk length 128) on the raw decay tensor of "
                          "--cfg 3 instead of the operators")
+    ap.add_argument("--edges", action="store_true",
+                    help="time the element-wise passes around the operator (token shift + mixing, ln_x * gate, channel-mix "
+                         "activations, L2Wrap backward) at the cfg3 and cfg4 shapes instead of the operator")
     ap.add_argument("--w-shift", type=float, default=0.0,
                     help="WKV6 only: added to the raw decay parameter (negative = slower decay; -5 makes every channel "
                          "remember for thousands of tokens, the worst case of the time-parallel split's summary passes)")
@@ -354,6 +357,82 @@ def bench_helper(a):
                       "dtype": "f32", "value": res["log_tables"]["ms"], "higher_is_better": False, "kernels": res}))
 
 
+def bench_edges(a):
+    """The element-wise passes around the operator (csrc/block_edges.hip), each kernel alone, bf16, at the token
+    counts and widths of cfg3 (B8 T4096 C2560) and cfg4 (B1 T4096 C4096).  Algorithmic bytes: every tensor the
+    reference's lines read or write, once (2 B per bf16 element; parameters are negligible).  Inputs and outputs
+    rotate over several sets so that nothing is served from the 256 MB last-level cache."""
+    import ctypes
+    import torch
+    from rwkv_wkv_hip import _lib
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    bf = torch.bfloat16
+    p = lambda t: None if t is None else t.data_ptr()
+    arr = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    res = {}
+
+    def timed(name, calls, nbytes):
+        for _ in range(max(a.warmup // 10, 2)):
+            for c in calls:
+                assert c() == 0
+        n = max(a.steps // 20, 5)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(n):
+            for c in calls:
+                c()
+        ev1.record()
+        torch.cuda.synchronize()
+        ms = ev0.elapsed_time(ev1) / (n * len(calls))
+        res[name] = {"ms": round(ms, 5), "algorithmic_bytes": nbytes, "GBs": round(nbytes / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    for tag, B, T, C in (("cfg3", 8, 4096, 2560), ("cfg4", 1, 4096, 4096)):
+        E = B * T * C
+        rot = 3 if tag == "cfg3" else 6
+        rnd = lambda *sh: torch.randn(*sh, device="cuda", dtype=bf)
+        sets = []
+        for _ in range(rot):
+            sets.append(dict(x=rnd(B, T, C), shift=rnd(B, C), dyn=rnd(5, B, T, C) * 0.3, o=[rnd(B, T, C) for _ in range(5)],
+                             gx=rnd(B, T, C), gshift=rnd(B, C), gdyn=torch.empty(5, B, T, C, device="cuda", dtype=bf)))
+        coef = torch.rand(5, C, device="cuda")
+        gcoef = torch.empty(5, C, device="cuda")
+        ws = torch.empty(max(L.wkv_shift_mix_backward_workspace(B, T, C, 5), L.wkv_ln_gate_backward_workspace(B * T, C)),
+                         dtype=torch.uint8, device="cuda")
+        wb, gwb = torch.randn(2, C, device="cuda"), torch.empty(2, C, device="cuda")
+        mk = lambda f: [(lambda s=s: f(s)) for s in sets]
+        timed(f"{tag} shift_mix v5 forward (4 mixes)", mk(lambda s: L.wkv_shift_mix_forward(
+            stream, B, T, C, 1, 4, 1, p(s["x"]), p(s["shift"]), p(coef), None, arr(s["o"][:4]))), 10 * E)
+        timed(f"{tag} shift_mix v5 backward (4 mixes)", mk(lambda s: L.wkv_shift_mix_backward(
+            stream, B, T, C, 1, 4, 1, p(s["x"]), p(s["shift"]), p(coef), None, arr(s["o"][:4]), p(s["gx"]), p(s["gshift"]), p(gcoef),
+            None, p(ws), ws.numel())), 12 * E)
+        timed(f"{tag} shift_mix v6 forward (5 mixes + data-dependent part)", mk(lambda s: L.wkv_shift_mix_forward(
+            stream, B, T, C, 1, 5, 0, p(s["x"]), p(s["shift"]), p(coef), p(s["dyn"]), arr(s["o"]))), 22 * E)
+        timed(f"{tag} shift_mix v6 backward (5 mixes + data-dependent part)", mk(lambda s: L.wkv_shift_mix_backward(
+            stream, B, T, C, 1, 5, 0, p(s["x"]), p(s["shift"]), p(coef), p(s["dyn"]), arr(s["o"]), p(s["gx"]), p(s["gshift"]), p(gcoef),
+            p(s["gdyn"]), p(ws), ws.numel())), 34 * E)
+        timed(f"{tag} ln_x * gate forward", mk(lambda s: L.wkv_ln_gate_forward(
+            stream, B * T, C, 1, 1.0, 64e-5, p(s["x"]), p(s["o"][0]), p(wb[0]), p(wb[1]), p(s["gx"]))), 6 * E)
+        timed(f"{tag} ln_x * gate backward", mk(lambda s: L.wkv_ln_gate_backward(
+            stream, B * T, C, 1, 1.0, 64e-5, p(s["x"]), p(s["o"][0]), p(wb[0]), p(wb[1]), p(s["o"][1]), p(s["gx"]), p(s["o"][2]),
+            p(gwb), p(ws), ws.numel())), 10 * E)
+        timed(f"{tag} relu^2 forward", mk(lambda s: L.wkv_relu_square_forward(stream, E, 1, p(s["x"]), p(s["gx"]))), 4 * E)
+        timed(f"{tag} relu^2 backward", mk(lambda s: L.wkv_relu_square_backward(stream, E, 1, p(s["x"]), p(s["o"][0]), p(s["gx"]))), 6 * E)
+        timed(f"{tag} sigmoid * kv forward", mk(lambda s: L.wkv_sigmoid_mul_forward(stream, E, 1, p(s["x"]), p(s["o"][0]), p(s["gx"]))), 6 * E)
+        timed(f"{tag} sigmoid * kv backward", mk(lambda s: L.wkv_sigmoid_mul_backward(
+            stream, E, 1, p(s["x"]), p(s["o"][0]), p(s["o"][1]), p(s["gx"]), p(s["o"][2]))), 10 * E)
+        del sets
+    rows, V = 4096, 65536
+    ys = [torch.randn(rows, V, device="cuda", dtype=bf) for _ in range(2)]
+    gys = [torch.empty_like(y) for y in ys]
+    timed("L2Wrap backward (4096 rows, vocabulary 65536)",
+          [(lambda i=i: L.wkv_l2wrap_backward(stream, rows, V, 1, 1e-4 / rows, p(ys[i]), None, p(gys[i]))) for i in range(2)], 4 * rows * V)
+    key = "cfg4 shift_mix v6 backward (5 mixes + data-dependent part)"
+    print(json.dumps({"metric": "element-wise passes around the WKV operator, bf16", "unit": "GB/s", "n_gpus": 1, "data": "synthetic",
+                      "dtype": "bf16", "value": res[key]["GBs"], "higher_is_better": True, "kernels": res}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -364,6 +443,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if a.helper:
         return bench_helper(a)
+    if a.edges:
+        return bench_edges(a)
     runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift, a.io_dtype)
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 

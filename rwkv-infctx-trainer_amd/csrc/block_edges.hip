@@ -173,20 +173,31 @@ __global__ __launch_bounds__(256) void shift_mix_backward(int Tlen, int C, int l
     }
 }
 
-// out[n] = sum over rows of in[row][n]; rows added in a fixed order (four interleaved running sums)
+// out[n] = sum over rows of in[row][n], rows added in a fixed order: 32 columns x 8 row groups per workgroup, each
+// group four interleaved running sums over its rows, the groups added in order at the end
 __global__ __launch_bounds__(256) void sum_rows(int rows, int n, const float *__restrict__ in, float *__restrict__ out) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
+    __shared__ float red[8][32];
+    const int lane = threadIdx.x & 31, rg = threadIdx.x >> 5;
+    const int i = blockIdx.x * 32 + lane;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    int r = 0;
-    for (; r + 4 <= rows; r += 4) {
-        s0 += in[(size_t)r * n + i];
-        s1 += in[(size_t)(r + 1) * n + i];
-        s2 += in[(size_t)(r + 2) * n + i];
-        s3 += in[(size_t)(r + 3) * n + i];
+    if (i < n) {
+        int r = rg;
+        for (; r + 24 < rows; r += 32) {
+            s0 += in[(size_t)r * n + i];
+            s1 += in[(size_t)(r + 8) * n + i];
+            s2 += in[(size_t)(r + 16) * n + i];
+            s3 += in[(size_t)(r + 24) * n + i];
+        }
+        for (; r < rows; r += 8) s0 += in[(size_t)r * n + i];
     }
-    for (; r < rows; r++) s0 += in[(size_t)r * n + i];
-    out[i] = (s0 + s1) + (s2 + s3);
+    red[rg][lane] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (rg == 0 && i < n) {
+        float s = red[0][lane];
+#pragma unroll
+        for (int g = 1; g < 8; g++) s += red[g][lane];
+        out[i] = s;
+    }
 }
 
 // ---- ln_x * gate
@@ -196,7 +207,11 @@ __device__ __forceinline__ float head_sum(float v) {          // over the 8 lane
     v += __shfl_xor(v, 4);
     return v;
 }
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + __expf(-x)); }
+// 1 / (1 + e^-x) on the hardware exp2 and reciprocal (1 ulp each): a full-precision division per element would make
+// these passes bound by vector instructions instead of by memory
+__device__ __forceinline__ float sigmoid_f(float x) { return __builtin_amdgcn_rcpf(1.f + exp2_fast(-LOG2E * x)); }
+
+constexpr int ROW_BATCH = 4;       // rows whose loads are issued together before any of them is used
 
 // out = (GroupNorm_head(y * scale) * weight + bias) * silu(gate); gate == nullptr: no gate
 template <class T>
@@ -210,34 +225,38 @@ __global__ __launch_bounds__(256) void ln_gate_forward(int rows, int C, float sc
     float w[8], bs[8];
     if (live) { load8(weight + c, w); load8(bias + c, bs); }
 #pragma unroll
-    for (int i = 0; i < ROWS_PER_LANE; i++) {
-        const int r = r0 + i;
-        if (r >= rows) break;                   // uniform over the 8 lanes of a head (same tl)
-        const size_t off = (size_t)r * C + c;
-        float v[8], g[8];
-        if (live) {
-            load8(y + off, v);
-            if (gate) load8(gate + off, g);
-        } else {
+    for (int i0 = 0; i0 < ROWS_PER_LANE; i0 += ROW_BATCH) {
+        float v[ROW_BATCH][8], g[ROW_BATCH][8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = 0.f;
+        for (int i = 0; i < ROW_BATCH; i++) {
+            const int r = r0 + i0 + i;
+#pragma unroll
+            for (int e = 0; e < 8; e++) { v[i][e] = 0.f; g[i][e] = 0.f; }
+            if (live && r < rows) {
+                load8(y + (size_t)r * C + c, v[i]);
+                if (gate) load8(gate + (size_t)r * C + c, g[i]);
+            }
         }
-        float s = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) { v[e] *= scale; s += v[e]; }
-        const float mean = head_sum(s) * (1.f / HEAD);
-        float q = 0.f;
+        for (int i = 0; i < ROW_BATCH; i++) {
+            const int r = r0 + i0 + i;
+            float s = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) { v[e] -= mean; q = fmaf(v[e], v[e], q); }
-        const float rstd = rsqrtf(head_sum(q) * (1.f / HEAD) + eps);
-        if (!live) continue;
-        float o[8];
+            for (int e = 0; e < 8; e++) { v[i][e] *= scale; s += v[i][e]; }
+            const float mean = head_sum(s) * (1.f / HEAD);
+            float q = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float n = fmaf(v[e] * rstd, w[e], bs[e]);
-            o[e] = gate ? n * g[e] * sigmoid_f(g[e]) : n;
+            for (int e = 0; e < 8; e++) { v[i][e] -= mean; q = fmaf(v[i][e], v[i][e], q); }
+            const float rstd = rsqrtf(head_sum(q) * (1.f / HEAD) + eps);
+            if (!live || r >= rows) continue;
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float n = fmaf(v[i][e] * rstd, w[e], bs[e]);
+                o[e] = gate ? n * g[i][e] * sigmoid_f(g[i][e]) : n;
+            }
+            store8(out + (size_t)r * C + c, o);
         }
-        store8(out + off, o);
     }
 }
 
@@ -256,50 +275,58 @@ __global__ __launch_bounds__(256) void ln_gate_backward(int rows, int C, float s
     for (int e = 0; e < 8; e++) { aw[e] = 0.f; ab[e] = 0.f; w[e] = 0.f; bs[e] = 0.f; }
     if (live) { load8(weight + c, w); load8(bias + c, bs); }
 #pragma unroll
-    for (int i = 0; i < ROWS_PER_LANE; i++) {
-        const int r = r0 + i;
-        if (r >= rows) break;
-        const size_t off = (size_t)r * C + c;
-        float v[8], g[8], go[8];
+    for (int i0 = 0; i0 < ROWS_PER_LANE; i0 += ROW_BATCH) {
+        float vv[ROW_BATCH][8], gg_[ROW_BATCH][8], go_[ROW_BATCH][8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) { v[e] = 0.f; g[e] = 0.f; go[e] = 0.f; }
-        if (live) {
-            load8(y + off, v);
-            load8(gout + off, go);
-            if (gate) load8(gate + off, g);
-        }
-        float s = 0.f;
+        for (int i = 0; i < ROW_BATCH; i++) {
+            const int r = r0 + i0 + i;
 #pragma unroll
-        for (int e = 0; e < 8; e++) { v[e] *= scale; s += v[e]; }
-        const float mean = head_sum(s) * (1.f / HEAD);
-        float q = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) { v[e] -= mean; q = fmaf(v[e], v[e], q); }
-        const float rstd = rsqrtf(head_sum(q) * (1.f / HEAD) + eps);
-        float gg[8], m1 = 0.f, m2 = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            v[e] *= rstd;                                       // normalised value
-            float gn = go[e];
-            if (gate) {
-                const float sg = sigmoid_f(g[e]), n = fmaf(v[e], w[e], bs[e]);
-                gg[e] = go[e] * n * sg * (1.f + g[e] * (1.f - sg));
-                gn = go[e] * g[e] * sg;
+            for (int e = 0; e < 8; e++) { vv[i][e] = 0.f; gg_[i][e] = 0.f; go_[i][e] = 0.f; }
+            if (live && r < rows) {
+                const size_t off = (size_t)r * C + c;
+                load8(y + off, vv[i]);
+                load8(gout + off, go_[i]);
+                if (gate) load8(gate + off, gg_[i]);
             }
-            aw[e] = fmaf(gn, v[e], aw[e]);
-            ab[e] += gn;
-            go[e] = gn * w[e];                                  // gradient of the normalised value
-            m1 += go[e];
-            m2 = fmaf(go[e], v[e], m2);
         }
-        m1 = head_sum(m1) * (1.f / HEAD);
-        m2 = head_sum(m2) * (1.f / HEAD);
-        if (!live) continue;
-        float o[8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = scale * rstd * (go[e] - m1 - v[e] * m2);
-        store8(gy + off, o);
-        if (gate) store8(ggate + off, gg);
+        for (int i = 0; i < ROW_BATCH; i++) {
+            const int r = r0 + i0 + i;
+            float (&v)[8] = vv[i], (&g)[8] = gg_[i], (&go)[8] = go_[i];
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) { v[e] *= scale; s += v[e]; }
+            const float mean = head_sum(s) * (1.f / HEAD);
+            float q = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) { v[e] -= mean; q = fmaf(v[e], v[e], q); }
+            const float rstd = rsqrtf(head_sum(q) * (1.f / HEAD) + eps);
+            float gg[8], m1 = 0.f, m2 = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                v[e] *= rstd;                                       // normalised value
+                float gn = go[e];
+                if (gate) {
+                    const float sg = sigmoid_f(g[e]), n = fmaf(v[e], w[e], bs[e]);
+                    gg[e] = go[e] * n * sg * (1.f + g[e] * (1.f - sg));
+                    gn = go[e] * g[e] * sg;
+                }
+                aw[e] = fmaf(gn, v[e], aw[e]);                      // rows past the end carry zeros
+                ab[e] += gn;
+                go[e] = gn * w[e];                                  // gradient of the normalised value
+                m1 += go[e];
+                m2 = fmaf(go[e], v[e], m2);
+            }
+            m1 = head_sum(m1) * (1.f / HEAD);
+            m2 = head_sum(m2) * (1.f / HEAD);
+            if (!live || r >= rows) continue;
+            const size_t off = (size_t)r * C + c;
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = scale * rstd * (go[e] - m1 - v[e] * m2);
+            store8(gy + off, o);
+            if (gate) store8(ggate + off, gg);
+        }
     }
 #pragma unroll
     for (int e = 0; e < 8; e++) { red[tl][0][cl * VEC + e] = aw[e]; red[tl][1][cl * VEC + e] = ab[e]; }
@@ -460,7 +487,7 @@ hipError_t shift_mix_backward_n(hipStream_t s, int B, int Tlen, int C, int lerp,
                        (const T *)shift, coef, (const T *)dyn, pg, (T *)gx, (T *)gshift, partial, (T *)gdyn);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(sum_rows, dim3((N * C + 255) / 256), dim3(256), 0, s, (int)(B * row_tiles(Tlen)), N * C, partial, gcoef);
+    hipLaunchKernelGGL(sum_rows, dim3((N * C + 31) / 32), dim3(256), 0, s, (int)(B * row_tiles(Tlen)), N * C, partial, gcoef);
     return hipGetLastError();
 }
 template <class T>
@@ -505,7 +532,7 @@ hipError_t ln_gate_backward_t(hipStream_t s, int rows, int C, float scale, float
                        (const T *)gate, weight, bias, (const T *)gout, (T *)gy, (T *)ggate, partial);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(sum_rows, dim3((2 * C + 255) / 256), dim3(256), 0, s, (int)row_tiles(rows), 2 * C, partial, gweight_gbias);
+    hipLaunchKernelGGL(sum_rows, dim3((2 * C + 31) / 32), dim3(256), 0, s, (int)row_tiles(rows), 2 * C, partial, gweight_gbias);
     return hipGetLastError();
 }
 

@@ -37,11 +37,6 @@ def _dtype_code(t):
     return _DT[t.dtype]
 
 
-def _param32(p, C):
-    """(.., C) parameter -> flat fp32 (C,) on the same device"""
-    return p.detach().reshape(-1).float().contiguous()
-
-
 class _ShiftMix(torch.autograd.Function):
     @staticmethod
     def forward(ctx, lerp, x, shift, coef, dyn):
