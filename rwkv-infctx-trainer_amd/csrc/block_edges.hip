@@ -16,9 +16,9 @@
 namespace wkv {
 namespace edges {
 
-constexpr int CH_LANES = 32, ROW_LANES = 8, VEC = 8, ROWS_PER_LANE = 8;
-constexpr int TILE_C = CH_LANES * VEC;                   // 256 channels per workgroup
-constexpr int TILE_R = ROW_LANES * ROWS_PER_LANE;        // 64 rows (tokens) per workgroup
+constexpr int CH_LANES = 64, ROW_LANES = 4, VEC = 8, ROWS_PER_LANE = 8;
+constexpr int TILE_C = CH_LANES * VEC;                   // channels per workgroup
+constexpr int TILE_R = ROW_LANES * ROWS_PER_LANE;        // rows (tokens) per workgroup
 constexpr int MAX_MIX = 5;
 
 template <class T> __device__ __forceinline__ void load8(const T *p, float (&o)[8]) {
