@@ -310,6 +310,7 @@ size_t wkv_shift_mix_backward_workspace(int B, int T, int C, int n) {
 int wkv_shift_mix_forward(void *stream, int B, int T, int C, int dtype, int n, int lerp, const void *x, const void *shift,
                           const float *coef, const void *dyn, void *const *out) {
     if (B <= 0 || T <= 0 || C <= 0 || C % 8 != 0 || B > 65535 || n <= 0 || n > edges::MAX_MIX) return WKV_ERR_DIMS;
+    if ((T + edges::TILE_R - 1) / edges::TILE_R > 65535) return WKV_ERR_DIMS;          // rows of workgroups in one launch
     if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
     if (!x || !shift || !coef || !out) return WKV_ERR_NULL;
     for (int j = 0; j < n; j++) {
@@ -328,6 +329,7 @@ int wkv_shift_mix_backward(void *stream, int B, int T, int C, int dtype, int n, 
                            const float *coef, const void *dyn, const void *const *gout, void *gx, void *gshift, float *gcoef,
                            void *gdyn, void *workspace, size_t workspace_bytes) {
     if (B <= 0 || T <= 0 || C <= 0 || C % 8 != 0 || B > 65535 || n <= 0 || n > edges::MAX_MIX) return WKV_ERR_DIMS;
+    if ((T + edges::TILE_R - 1) / edges::TILE_R > 65535) return WKV_ERR_DIMS;          // rows of workgroups in one launch
     if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
     if (!x || !shift || !coef || !gout || !gx || !gshift || !gcoef || !workspace || (dyn && !gdyn)) return WKV_ERR_NULL;
     for (int j = 0; j < n; j++) {
