@@ -58,6 +58,9 @@ def parse():
     ap.add_argument("--edges", action="store_true",
                     help="time the element-wise passes around the operator (token shift + mixing, ln_x * gate, channel-mix "
                          "activations, L2Wrap backward) at the cfg3 and cfg4 shapes instead of the operator")
+    ap.add_argument("--block", action="store_true",
+                    help="time one whole RWKV-v6 TimeMix + ChannelMix layer (cfg4 width, fwd+bwd): element-wise passes on the "
+                         "HIP kernels against the same layer with torch element-wise ops around the same WKV operator")
     ap.add_argument("--w-shift", type=float, default=0.0,
                     help="WKV6 only: added to the raw decay parameter (negative = slower decay; -5 makes every channel "
                          "remember for thousands of tokens, the worst case of the time-parallel split's summary passes)")
@@ -433,6 +436,103 @@ def bench_edges(a):
                       "dtype": "bf16", "value": res[key]["GBs"], "higher_is_better": True, "kernels": res}))
 
 
+def bench_block(a):
+    """One RWKV-v6 layer's TimeMix and ChannelMix (RWKV-v6/src/module/TimeMix.py:253-302, ChannelMix.py:30-37) at the
+    cfg4 width (B1 T4096 C4096 H64, dim_ffn 14336, bf16), forward + backward, two ways: every element-wise pass on the
+    HIP kernels (rwkv_wkv_hip.blocks), and the same layer written with torch element-wise ops as the reference writes
+    it.  Both use the same WKV6 operator and the same torch matmuls, so the difference is the element-wise passes."""
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import blocks as K
+    B, T, C, H, FFN = 1, 4096, 4096, 64, 14336
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device="cpu").manual_seed(5)
+
+    class TimeMix(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.n_head = H
+            u01 = lambda *sh: torch.rand(*sh, generator=g)
+            for nm in ("x", "w", "k", "v", "r", "g"):
+                setattr(self, f"time_maa_{nm}", nn.Parameter(u01(1, 1, C)))
+            self.time_maa_w1 = nn.Parameter((u01(C, 160) - 0.5) * 0.02)
+            self.time_maa_w2 = nn.Parameter((u01(5, 32, C) - 0.5) * 0.02)
+            self.time_decay = nn.Parameter(u01(1, 1, C) * 5 - 6)
+            self.time_decay_w1 = nn.Parameter((u01(C, 64) - 0.5) * 0.02)
+            self.time_decay_w2 = nn.Parameter((u01(64, C) - 0.5) * 0.02)
+            self.time_faaaa = nn.Parameter(torch.randn(H, 64, generator=g) * 0.3)
+            self.receptance, self.key, self.value, self.gate, self.output = (nn.Linear(C, C, bias=False) for _ in range(5))
+            self.ln_x = nn.GroupNorm(H, C, eps=64e-5)
+
+    class ChannelMix(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.time_maa_k = nn.Parameter(torch.rand(1, 1, C, generator=g))
+            self.time_maa_r = nn.Parameter(torch.rand(1, 1, C, generator=g))
+            self.key, self.receptance, self.value = nn.Linear(C, FFN, bias=False), nn.Linear(C, C, bias=False), nn.Linear(FFN, C, bias=False)
+
+    def timemix_torch(m, x, st):            # the reference's lines, element-wise work in torch
+        dxprev = torch.concat((st[0].unsqueeze(1), x[:, :-1]), dim=1) - x
+        xxx = x + dxprev * m.time_maa_x
+        xxx = torch.tanh(xxx @ m.time_maa_w1).view(B * T, 5, -1).transpose(0, 1)
+        mw, mk, mv, mr, mg = torch.bmm(xxx, m.time_maa_w2).view(5, B, T, -1).unbind(dim=0)
+        xk, xv, xr = x + dxprev * (m.time_maa_k + mk), x + dxprev * (m.time_maa_v + mv), x + dxprev * (m.time_maa_r + mr)
+        xg, xw = x + dxprev * (m.time_maa_g + mg), x + dxprev * (m.time_maa_w + mw)
+        r, k, v, gate = m.receptance(xr), m.key(xk), m.value(xv), F.silu(m.gate(xg))
+        w = m.time_decay + torch.tanh(xw @ m.time_decay_w1) @ m.time_decay_w2
+        y, ns = W.WKV_6.apply(B, T, C, H, r, k, v, w.contiguous(), m.time_faaaa, st[1])
+        y = m.ln_x(y.view(-1, C)).view(B, T, C)
+        return m.output(y * gate), (x[:, -1], ns)
+
+    def channelmix_torch(m, x, st):
+        dxx = torch.concat((st.unsqueeze(1), x[:, :-1]), dim=1) - x
+        xk, xr = x + dxx * m.time_maa_k, x + dxx * m.time_maa_r
+        kv = m.value(torch.relu(m.key(xk)) ** 2)
+        return torch.sigmoid(m.receptance(xr)) * kv, x[:, -1]
+
+    tm, cm = TimeMix().to(dev).to(bf), ChannelMix().to(dev).to(bf)
+    x = (torch.randn(B, T, C, generator=g) * 0.5).to(dev).to(bf).requires_grad_(True)
+    shift = torch.randn(B, C, generator=g).to(dev).to(bf)
+    state = (torch.randn(B, H, 64, 64, generator=g) * 0.1).to(dev)
+    gy = torch.randn(B, T, C, generator=g).to(dev).to(bf)
+    res = {}
+
+    def timed(name, fn):
+        def once():
+            x.grad = None
+            for p in list(tm.parameters()) + list(cm.parameters()):
+                p.grad = None
+            y = fn()
+            y.backward(gy)
+        for _ in range(3):
+            once()
+        n = max(a.steps // 30, 10)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(n):
+            once()
+        ev1.record()
+        torch.cuda.synchronize()
+        res[name] = round(ev0.elapsed_time(ev1) / n, 4)
+    timed("timemix_kernels_ms", lambda: K.timemix6_forward(tm, x, (shift, state))[0])
+    timed("timemix_torch_elementwise_ms", lambda: timemix_torch(tm, x, (shift, state))[0])
+    timed("channelmix_kernels_ms", lambda: K.channelmix6_forward(cm, x, shift)[0])
+    timed("channelmix_torch_elementwise_ms", lambda: channelmix_torch(cm, x, shift)[0])
+    with torch.no_grad():       # the two ways agree
+        ya, yb = K.timemix6_forward(tm, x, (shift, state))[0].float(), timemix_torch(tm, x, (shift, state))[0].float()
+        res["timemix_rel_diff"] = round(((ya - yb).norm() / yb.norm()).item(), 5)
+        ya, yb = K.channelmix6_forward(cm, x, shift)[0].float(), channelmix_torch(cm, x, shift)[0].float()
+        res["channelmix_rel_diff"] = round(((ya - yb).norm() / yb.norm()).item(), 5)
+    layer_k = res["timemix_kernels_ms"] + res["channelmix_kernels_ms"]
+    layer_t = res["timemix_torch_elementwise_ms"] + res["channelmix_torch_elementwise_ms"]
+    print(json.dumps({"metric": "RWKV-v6 layer (TimeMix + ChannelMix) fwd+bwd, B1 T4096 C4096 H64 bf16, host-launched (autograd)", "unit": "ms",
+                      "n_gpus": 1, "data": "synthetic", "dtype": "bf16", "value": round(layer_k, 4), "higher_is_better": False,
+                      "torch_elementwise_ms": round(layer_t, 4), "speedup": round(layer_t / layer_k, 3), "parts": res}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -445,6 +545,8 @@ def main():
         return bench_helper(a)
     if a.edges:
         return bench_edges(a)
+    if a.block:
+        return bench_block(a)
     runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift, a.io_dtype)
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
