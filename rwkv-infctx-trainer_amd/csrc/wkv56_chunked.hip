@@ -882,7 +882,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     }
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};      // block phase: this lane's token, keys 16wv+4g..+3
     const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + 16 * wv + 4 * g);      // the bonus of those keys
-    float4 gw_acc = make_float4(0.f, 0.f, 0.f, 0.f);      // time-invariant w: sum over this lane's tokens, channels c4..c4+3
+    // Time-invariant w: its gradient is the SUM over tokens of dL/dlog w_t = A_t - z_t, A_t = A(segment end) + sum_{s>t} c_s,
+    // and  sum_t A_t = (tokens) A(segment end) + sum_s (tokens before s) c_s:  no running sum, no per-token values, just
+    // one weighted sum per lane (block phase: this lane's token, keys 16wv+4g..+3).
+    float gw_acc[4] = {0.f, 0.f, 0.f, 0.f};
 
     // preparing role: token tok of the step (block q), channels c4..c4+3 (one 128-byte row per 16 lanes)
     const int c4 = 4 * n, tok = 4 * w16 + g;
@@ -911,6 +914,15 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     // the first being the sum at the step's end (arun[par]) plus the totals of the step's later blocks.
     auto write_out = [&](int sb, int tok, int c4, int par) {
         const int t = sb * SB + tok;
+        if (!PER_TOKEN_W) {         // nothing per token to finish: gr, gk, gv only
+            if (t < Tlen) {
+                const size_t o = base + (size_t)t * C + c4;
+                *reinterpret_cast<uint2 *>(gr + o) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
+                *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
+                *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
+            }
+            return;
+        }
         float4 A = *reinterpret_cast<const float4 *>(&sm.arun[par][c4]);
         const float4 t1 = *reinterpret_cast<const float4 *>(&sm.tots[1][c4]), t2 = *reinterpret_cast<const float4 *>(&sm.tots[2][c4]);
         const float4 t3 = *reinterpret_cast<const float4 *>(&sm.tots[3][c4]);
@@ -932,7 +944,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             *reinterpret_cast<uint2 *>(gr + o) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
             *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
             *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
-            if (PER_TOKEN_W) {      // dL/dw_raw = dL/dlog w x log w (natural logarithm); nothing where the floor holds
+            {                       // dL/dw_raw = dL/dlog w x log w (natural logarithm); nothing where the floor holds
                 const float4 l4 = *reinterpret_cast<const float4 *>(&sm.lw[swz(tok, c4)]);
                 const float lf[4] = {l4.x, l4.y, l4.z, l4.w};
                 float f[4];
@@ -941,8 +953,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                 const float gw4[4] = {A.x * f[0], A.y * f[1], A.z * f[2], A.w * f[3]};
                 if (W16) store4(static_cast<bf16 *>(gw_tok) + o, gw4);
                 else store4(static_cast<float *>(gw_tok) + o, gw4);
-            } else {
-                gw_acc.x += A.x; gw_acc.y += A.y; gw_acc.z += A.z; gw_acc.w += A.w;
             }
         }
     };
@@ -1262,17 +1272,23 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             // this wavefront was the only reader left of its (block, quarter) corner of the rh and kh tiles
             *reinterpret_cast<uint2 *>(&sm.rh[tk * LD + k4]) = make_uint2(bf16_pack2(grv[0], grv[1]), bf16_pack2(grv[2], grv[3]));
             *reinterpret_cast<uint2 *>(&sm.kh[tk * LD + k4]) = make_uint2(bf16_pack2(gkv[0], gkv[1]), bf16_pack2(gkv[2], gkv[3]));
-            // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over the block's later tokens of c
-            float dpart[4], all[4];
+            if (PER_TOKEN_W) {
+                // dL/dlog w_t = A_t - z_t with A_t = A(end of block) + sum over the block's later tokens of c
+                float dpart[4], all[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float incl_suf = row_suffix_sum(c[e]);          // c of this token and the later ones
-                dpart[e] = (incl_suf - c[e]) - z[e];
-                all[e] = incl_suf;                                    // (lane n = 0: the whole block)
+                for (int e = 0; e < 4; e++) {
+                    const float incl_suf = row_suffix_sum(c[e]);          // c of this token and the later ones
+                    dpart[e] = (incl_suf - c[e]) - z[e];
+                    all[e] = incl_suf;                                    // (lane n = 0: the whole block)
+                }
+                // (the incl entries of this block and quarter had this wavefront as their only reader)
+                *reinterpret_cast<float4 *>(&sm.incl[ti]) = make_float4(dpart[0], dpart[1], dpart[2], dpart[3]);
+                if (n == 0) *reinterpret_cast<float4 *>(&sm.tots[q][k4]) = make_float4(all[0], all[1], all[2], all[3]);
+            } else {
+                const float before = (float)((sb - sb0) * SB + tk);      // tokens of the segment before this one
+#pragma unroll
+                for (int e = 0; e < 4; e++) gw_acc[e] += fmaf(before, c[e], -z[e]);
             }
-            // (the incl entries of this block and quarter had this wavefront as their only reader)
-            *reinterpret_cast<float4 *>(&sm.incl[ti]) = make_float4(dpart[0], dpart[1], dpart[2], dpart[3]);
-            if (n == 0) *reinterpret_cast<float4 *>(&sm.tots[q][k4]) = make_float4(all[0], all[1], all[2], all[3]);
         }
       }
         PT_MARK(4)
@@ -1291,11 +1307,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
     for (int e = 0; e < 4; e++) gu_acc[e] = row_suffix_sum(gu_acc[e]);       // lane n = 0: the sum over the row's 16 tokens
     if (n == 0) *reinterpret_cast<float4 *>(&sm.red[q][16 * wv + 4 * g]) = make_float4(gu_acc[0], gu_acc[1], gu_acc[2], gu_acc[3]);
-    float *gw16 = sm.q1;            // [16][HEAD]; the q1 table is dead by now
+    float *gw4 = sm.q1;             // [4][HEAD]; the q1 table is dead by now
     if (!PER_TOKEN_W) {
-        gw_acc.x = group_sum4(gw_acc.x); gw_acc.y = group_sum4(gw_acc.y);
-        gw_acc.z = group_sum4(gw_acc.z); gw_acc.w = group_sum4(gw_acc.w);
-        if (g == 0) *reinterpret_cast<float4 *>(&gw16[w16 * HEAD + c4]) = gw_acc;
+#pragma unroll
+        for (int e = 0; e < 4; e++) gw_acc[e] = row_suffix_sum(gw_acc[e]);
+        if (n == 0) *reinterpret_cast<float4 *>(&gw4[q * HEAD + 16 * wv + 4 * g]) = make_float4(gw_acc[0], gw_acc[1], gw_acc[2], gw_acc[3]);
     }
     lds_barrier();
     if (q == 0 && g == 0) {      // partial sums per (batch, segment): [(b*nseg + seg)][C]
@@ -1304,9 +1320,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         if (!PER_TOKEN_W) {
             bool fl;
             const float l = log_decay(static_cast<const float *>(wraw)[h * HEAD + own], floor_decay, &fl);
-            float sum = 0.f;
-#pragma unroll
-            for (int x = 0; x < 16; x++) sum += gw16[x * HEAD + own];
+            const int ntok = min(Tlen, sb1 * SB) - sb0 * SB;         // tokens of this segment
+            const float sum = ((gw4[own] + gw4[HEAD + own]) + (gw4[2 * HEAD + own] + gw4[3 * HEAD + own]))
+                              + (float)ntok * sm.arun[0][own];            // arun[0]: the anchor A(segment end), untouched for this w
             gw_part[po] = fl ? 0.f : sum * l;
         }
     }
