@@ -181,6 +181,43 @@ def test_timemix_forward_on_the_kernels(version, T):
 
 
 @pytest.mark.parametrize("version", [5, 6])
+def test_timemix_forward_on_the_kernels_bf16_module(version):
+    """The whole module in bf16 (weights, matmuls, every element-wise pass), as mixed-precision training runs it, against
+    the fp32 CPU module: compared in norm (the matmuls round too); the carried state, which only the operator touches and
+    which stays fp32, element-wise."""
+    from rwkv_wkv_hip import blocks as K
+    B, T, C, H = 2, 128, 128, 2
+    g = _g(13)
+    x, shift = torch.randn(B, T, C, generator=g), torch.randn(B, C, generator=g)
+    state = torch.randn(B, H, 64, 64, generator=g) * 0.1
+    gy = torch.randn(B, T, C, generator=g)
+    cpu = (TimeMix5 if version == 5 else TimeMix6)(C, H, seed=8)
+    gpu = copy.deepcopy(cpu).cuda().bfloat16()
+    if version == 5:
+        ref_fwd = lambda m, xs, st: m(xs, st, lambda B, T, C, H, s, r, k, v, w, u: O.wkv5_op(B, T, C, H, s, r, k, v, w, u))
+        our_fwd = K.timemix5_forward
+    else:
+        ref_fwd = lambda m, xs, st: m(xs, st, lambda B, T, C, H, r, k, v, w, u, s: O.wkv6_op(B, T, C, H, r, k, v, w, u, s))
+        our_fwd = K.timemix6_forward
+    ref = _run_module(ref_fwd, cpu, x, (shift, state), gy)
+    got = _run_module(our_fwd, gpu, x.cuda().bfloat16(), (shift.cuda().bfloat16(), state.cuda()), gy.cuda().bfloat16())
+    torch.cuda.synchronize()
+    assert got[0].dtype == torch.bfloat16
+    for name, a, b in zip(("y", "gx", "gshift"), got[:3], ref[:3]):
+        rel = ((a.float().cpu() - b).norm() / b.norm()).item()
+        assert rel < 4e-2, f"timemix bf16 v{version} {name}: relative error {rel}"
+    for n in ref[3]:
+        a, b = got[3][n], ref[3][n]
+        rel = ((a - b).norm() / (b.norm() + 1e-6)).item()
+        assert rel < 8e-2, f"timemix bf16 v{version} grad {n}: relative error {rel}"
+    with torch.no_grad():
+        _, (_, s_ref) = ref_fwd(cpu, x, (shift, state))
+        _, (_, s_got) = our_fwd(gpu, x.cuda().bfloat16(), (shift.cuda().bfloat16(), state.cuda()))
+    assert s_got.dtype == torch.float32
+    assert_close(s_got, s_ref, 6e-2, f"timemix bf16 v{version} state")
+
+
+@pytest.mark.parametrize("version", [5, 6])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_channelmix_forward_on_the_kernels(version, dtype):
     from rwkv_wkv_hip import blocks as K
