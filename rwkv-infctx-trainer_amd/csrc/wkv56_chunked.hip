@@ -136,6 +136,17 @@ template <> struct WReg<false> {
     static __device__ __forceinline__ WReg load(const void *w, size_t o) {
         return WReg{*reinterpret_cast<const float4 *>(static_cast<const float *>(w) + o)};
     }
+    // The same as two 8-byte loads, for a value that stays in flight across a phase short of registers: a 16-byte load
+    // wants four consecutive registers, which the allocator there gives only at the price of copies that wait for the
+    // load on the spot.
+    static __device__ __forceinline__ WReg load_in_halves(const void *w, size_t o) {
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        size_t o2 = o + 2;
+        asm volatile("" : "+v"(o2));          // (opaque: the two loads are not seen to be adjacent, so they are not merged)
+        const f2 a = *reinterpret_cast<const f2 *>(static_cast<const float *>(w) + o);
+        const f2 b = *reinterpret_cast<const f2 *>(static_cast<const float *>(w) + o2);
+        return WReg{make_float4(a[0], a[1], b[0], b[1])};
+    }
     static __device__ __forceinline__ WReg from(float4 x) { return WReg{x}; }
     __device__ __forceinline__ float4 f4() const { return v; }
 };
@@ -144,10 +155,17 @@ template <> struct WReg<true> {
     static __device__ __forceinline__ WReg load(const void *w, size_t o) {
         return WReg{*reinterpret_cast<const uint2 *>(static_cast<const bf16 *>(w) + o)};
     }
+    static __device__ __forceinline__ WReg load_in_halves(const void *w, size_t o) { return load(w, o); }
     static __device__ __forceinline__ WReg from(float4 x) { return WReg{make_uint2(bf16_pack2(x.x, x.y), bf16_pack2(x.z, x.w))}; }
     __device__ __forceinline__ float4 f4() const { return make_float4(bf_lo(v.x), bf_hi(v.x), bf_lo(v.y), bf_hi(v.y)); }
 };
 #define WKV_NEG_INF4 make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY)
+// "These registers are needed HERE": makes the compiler wait for the loads that fill them at this point.  One counter
+// covers a wavefront's loads and stores, and a wait the compiler places after a conditional memory operation is
+// counted for the path without it: a wait for the step's inputs placed after the (conditional) result stores would
+// also wait for those stores to complete.
+__device__ __forceinline__ void needed_here(uint2 &a) { asm volatile("" : "+v"(a.x), "+v"(a.y)); }
+__device__ __forceinline__ void needed_here(float4 &a) { asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w)); }
 
 // One segment's summary for the time-parallel split: what the segment does to a
 // state handed in, S_out = decay o S_in + delta (forward), or to a state gradient
@@ -790,6 +808,7 @@ struct Bwd16Tiles {
     float dec[4][HEAD];      // e^{b}
     float ent[4][HEAD];      // e^{-b}
     float rho[SB];           // r . (u o k) per token
+    float ub[HEAD];
     float wtot[16][HEAD];    // per wavefront (four tokens) and channel: sum of log w, for the block-wide running sum
     float q1[SB * HEAD];     // gy S^T          [token][key]
     float q4[SB * HEAD];     // v G^T           [token][key]
@@ -907,6 +926,17 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             if (PER_TOKEN_W) pw = WReg<W16>::from(WKV_NEG_INF4);
         }
     };
+    // the same without a branch (the token clamped into the sequence): for the fetches inside the step loop, whose steps
+    // are whole; a wait the compiler places after a conditional load is counted for the path without it
+    auto fetch_whole = [&](int sb, int tok, int c4) {
+        const int t = min(sb * SB + tok, Tlen - 1);
+        const size_t o = base + (size_t)t * C + c4;
+        pr = *reinterpret_cast<const uint2 *>(r + o);
+        pk = *reinterpret_cast<const uint2 *>(k + o);
+        pv = *reinterpret_cast<const uint2 *>(v + o);
+        pg = *reinterpret_cast<const uint2 *>(gy + o);
+        if (PER_TOKEN_W) pw = WReg<W16>::load_in_halves(wraw, o);
+    };
     const int lane0 = lane;
     // gr, gk, gv of a finished step wait in the rh, kh, v tiles, [token][channel]; they leave as full rows, written
     // by the lanes that overwrite those entries next.  The decay gradient is finished on the way out:
@@ -968,6 +998,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     auto whole_step = [&](int sb) { return !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
 
     fetch(sb1 - 1, tok, c4);
+    if (tid < HEAD) sm.ub[tid] = u[h * HEAD + tid];
+    lds_barrier();
     PT_DECL
     for (int sb = sb1 - 1; sb >= sb0; sb--) {
       PT_MARK(5)
@@ -988,6 +1020,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
       if (!whole) tables_valid = false;
       {
         WKV_LOCAL_LANE
+        needed_here(pr); needed_here(pk); needed_here(pv); needed_here(pg);
+        if (PER_TOKEN_W) needed_here(pw.v);
         // the step's checkpoint: loads issued now are back when the chains start
         if (role == 0) {
             const float *ck_lane = ckpt + (size_t)bh * (nsb + 1) * HEAD * HEAD + (wv * 64 + 16 * (n >> 2) + 4 * g) * 4 + (n & 3);
@@ -1003,7 +1037,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             float l[4] = {pf.x, pf.y, pf.z, pf.w}, inc[4], tot[4];
             const float rf[4] = {bf_lo(pr.x), bf_hi(pr.x), bf_lo(pr.y), bf_hi(pr.y)};
             const float kf[4] = {bf_lo(pk.x), bf_hi(pk.x), bf_lo(pk.y), bf_hi(pk.y)};
-            const float4 u4 = *reinterpret_cast<const float4 *>(u + h * HEAD + c4);
+            const float4 u4 = *reinterpret_cast<const float4 *>(&sm.ub[c4]);
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
             if (PER_TOKEN_W) {
 #pragma unroll
@@ -1071,6 +1105,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         f4 KG[4];                    // wavefronts 8-11: kh G per block, KG[q][e] at [token 4g+e][value own]
       {
         WKV_LOCAL_LANE
+        fetch_whole(max(sb - 1, sb0), tok, c4);      // (the segment's first step fetches itself once more: unused)
         if (role == 0) {
             // ---------------- state chain, first block to last; Q1[t][key own] = sum_j gy[t][j] S[key own][j]
 #pragma unroll
@@ -1205,7 +1240,6 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             split2(at[0], at[1], h0, l0); split2(at[2], at[3], h1, l1);
             sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
         }
-        if (sb > sb0) fetch(sb - 1, tok, c4);      // after the chains: they are short of registers
       }
         PT_MARK(2)
         lds_barrier();
