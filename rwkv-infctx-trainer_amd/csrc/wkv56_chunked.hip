@@ -121,6 +121,17 @@ __device__ __forceinline__ void scale_split(s4 hi, s4 lo, float4 f, bool zero, s
     oh = as_s4(h0, h1);
     ol = as_s4(l0, l1);
 }
+// Result rows leave with the non-temporal hint: they are not read again by these kernels, and left to the default
+// policy they push the inputs that the backward pass reads a second time out of the last-level cache.
+__device__ __forceinline__ void store_row(bf16 *p, uint2 v) {
+    typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+    __builtin_nontemporal_store(u2{v.x, v.y}, reinterpret_cast<u2 *>(p));
+}
+__device__ __forceinline__ void store_row(bf16 *p, const float (&x)[4]) { store_row(p, make_uint2(bf16_pack2(x[0], x[1]), bf16_pack2(x[2], x[3]))); }
+__device__ __forceinline__ void store_row(float *p, const float (&x)[4]) {
+    typedef float f4_ __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(f4_{x[0], x[1], x[2], x[3]}, reinterpret_cast<f4_ *>(p));
+}
 __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane groups of 16
     x += __shfl_xor(x, 16);
     x += __shfl_xor(x, 32);
@@ -220,9 +231,9 @@ __device__ __forceinline__ float row_suffix_sum(float x) {
 }
 // Index into a [token][64 keys] fp32 table of the backward kernel.  The tables are written one token row per 16 lanes
 // (four keys a lane) by the preparing lanes and read one token per lane (four keys) by the block phase; without the
-// exchange of 16-byte pieces inside 128-byte groups by the row number, the second pattern would put eight lanes on
-// the same banks.
-__device__ __forceinline__ int swz(int row, int col) { return row * HEAD + (col ^ ((row & 7) << 2)); }
+// exchange of 16-byte pieces inside a row by the row number, the second pattern would put the sixteen lanes of a group
+// (sixteen consecutive rows, the same columns) on the same banks.
+__device__ __forceinline__ int swz(int row, int col) { return row * HEAD + (col ^ ((row & 15) << 2)); }
 // Transposing 8-byte LDS read: with every lane (g, a) of a 16-lane group pointing at
 // tile[row0 + 4g + a/4][col0 + 4(a%4) ..+3], lane (g, n) receives tile[row0 + 4g + i][col0 + n], i = 0..3:
 // an MFMA operand fragment with the rows along the contraction.  `off` = the lane's share of the address.
@@ -614,7 +625,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
             if (have_y) {      // y of the previous step waits in the rh tile: out as full rows, by the lanes that overwrite it next
                 const int t = (sb - 1) * SB + tok;
-                if (t < Tlen) *reinterpret_cast<uint2 *>(y + base + (size_t)t * C + c4) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
+                if (t < Tlen) store_row(y + base + (size_t)t * C + c4, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
             }
             const bool whole = whole_step(sb);
             float rhv[4], khv[4], p = 0.f;
@@ -738,7 +749,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     }
     if (have_y) {
         const int t = (sb1 - 1) * SB + tok;
-        if (t < Tlen) *reinterpret_cast<uint2 *>(y + base + (size_t)t * C + c4) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
+        if (t < Tlen) store_row(y + base + (size_t)t * C + c4, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
     }
     PT_PRINT("fwd16")
     if (chain && seg == nseg - 1) {
@@ -947,9 +958,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         if (!PER_TOKEN_W) {         // nothing per token to finish: gr, gk, gv only
             if (t < Tlen) {
                 const size_t o = base + (size_t)t * C + c4;
-                *reinterpret_cast<uint2 *>(gr + o) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
-                *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
-                *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
+                store_row(gr + o, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
+                store_row(gk + o, *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]));
+                store_row(gv + o, *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]));
             }
             return;
         }
@@ -971,9 +982,9 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         A.x += D.x; A.y += D.y; A.z += D.z; A.w += D.w;
         if (t < Tlen) {
             const size_t o = base + (size_t)t * C + c4;
-            *reinterpret_cast<uint2 *>(gr + o) = *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]);
-            *reinterpret_cast<uint2 *>(gk + o) = *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]);
-            *reinterpret_cast<uint2 *>(gv + o) = *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]);
+            store_row(gr + o, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
+            store_row(gk + o, *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]));
+            store_row(gv + o, *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]));
             {                       // dL/dw_raw = dL/dlog w x log w (natural logarithm); nothing where the floor holds
                 const float4 l4 = *reinterpret_cast<const float4 *>(&sm.lw[swz(tok, c4)]);
                 const float lf[4] = {l4.x, l4.y, l4.z, l4.w};
@@ -981,8 +992,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
                 for (int c = 0; c < 4; c++) f[c] = (floor_decay && lf[c] <= LOG2_W_FLOOR) ? 0.f : lf[c] * LN2;
                 const float gw4[4] = {A.x * f[0], A.y * f[1], A.z * f[2], A.w * f[3]};
-                if (W16) store4(static_cast<bf16 *>(gw_tok) + o, gw4);
-                else store4(static_cast<float *>(gw_tok) + o, gw4);
+                if (W16) store_row(static_cast<bf16 *>(gw_tok) + o, gw4);
+                else store_row(static_cast<float *>(gw_tok) + o, gw4);
             }
         }
     };
