@@ -9,7 +9,14 @@ is one forward + one backward call through the C ABI with all inputs resident
 in HBM.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--cfg 1|2|3|4] [--algo auto|recurrent|chunked]
-                    [--launch graph|eager]
+                    [--launch graph|eager] [--no-extras]
+
+Besides the line's own figures (``value``, ``ms_per_step``: the workload as BASELINE.json states it) the default run
+times the same K steps two more ways and reports them under their own keys: ``slow_decay`` (WKV6: the raw decay
+shifted by -5, i.e. no channel forgets inside a segment, which is what a freshly initialised RWKV-v6 layer looks
+like and the worst case of the time split's summary passes) and ``cold`` (the backward call of a segment runs two
+steps after its forward call, with other segments' calls in between, so that nothing it reads is still in the
+last-level cache: what a training step with a whole layer stack between forward and backward sees).
 
 The K timed steps are launched from HIP graphs (one graph of K steps up to
 K = 128; beyond that a 120-step body replayed K // 120 times plus one graph with
@@ -68,6 +75,10 @@ def parse():
                     help="untimed replays of the captured steps for this long before the timed region (the first replays "
                          "of a fresh graph run ~8 %% slower than the steady state a long run measures)")
     ap.add_argument("--segments", type=int, default=0, help="force the number of parallel time segments (0 = auto)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the slow-decay and cold-cache measurements of the default run")
+    ap.add_argument("--cold", action="store_true",
+                    help="make the cold-cache order (backward of the segment two steps back, then forward of this step's) the "
+                         "one that value / ms_per_step report")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run three plain 256 MiB device copies first (reference point for the FETCH_SIZE / "
                          "WRITE_SIZE counters of a profiler run)")
@@ -110,12 +121,15 @@ class Runner56:
         self.gw = torch.empty_like(s0["w"])
         self.gu = torch.empty_like(s0["u"])
         self.state = [s0["state"].clone(), torch.empty_like(s0["state"])]
-        self.gstate_in = torch.empty_like(s0["state"])
+        # the state gradient a backward call hands back is the one the next step's backward call is given
+        self.gstate = [s0["dstate"].clone(), torch.empty_like(s0["state"])]
         L = self.L
         q = (L.wkv5_forward_workspace, L.wkv5_backward_workspace) if self.version == 5 else \
             (L.wkv6_forward_workspace, L.wkv6_backward_workspace)
         nws = max(q[0](B, T, C, H, self.dt, self.algo), q[1](B, T, C, H, self.dt, self.algo), 16)
         self.ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+        self.ws_cold = None                             # second workspace, cold-cache order only
+        self.have_ckpt = q[0](B, T, C, H, self.dt, self.algo) > 0      # the forward call leaves its checkpoints in the workspace
         self.fwd = L.wkv5_forward if self.version == 5 else L.wkv6_forward
         self.bwd = L.wkv5_backward if self.version == 5 else L.wkv6_backward
         self.stream = torch.cuda.current_stream().cuda_stream
@@ -135,22 +149,47 @@ class Runner56:
                      f"{'bf16' if self.w16 else 'fp32'} raw decay, fp32 state, state carried step to step, state "
                      f"gradient fed back" + (f", raw decay shifted by {w_shift}" if w_shift else ""))
 
-    def step(self):
+    def _forward(self, s, s_in, s_out, ws):
         B, T, C, H = self.dims
-        s = self.sets[self.i % len(self.sets)]
-        s_in, s_out = self.state[self.i % 2], self.state[(self.i + 1) % 2]
-        self.i += 1
         p = lambda t: t.data_ptr()
         flags = self._lib.FLOOR_DECAY | (self._lib.W_BF16 if self.w16 else 0)
         st = self.fwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
-                      p(s["u"]), p(s_in), p(self.y), p(s_out), p(self.ws), self.ws.numel())
+                      p(s["u"]), p(s_in), p(self.y), p(s_out), p(ws), ws.numel())
         assert st == 0, self.L.wkv_strerror(st)
-        if self.L.wkv6_forward_workspace(B, T, C, H, self.dt, self.algo) > 0:
-            flags |= self._lib.CHECKPOINTS_VALID      # forward left its checkpoints in self.ws
+
+    def _backward(self, s, s_in, g_out, g_in, ws):
+        B, T, C, H = self.dims
+        p = lambda t: t.data_ptr()
+        flags = self._lib.FLOOR_DECAY | (self._lib.W_BF16 if self.w16 else 0)
+        if self.have_ckpt:
+            flags |= self._lib.CHECKPOINTS_VALID
         st = self.bwd(self.stream, B, T, C, H, self.dt, flags, self.algo, p(s["r"]), p(s["k"]), p(s["v"]), p(s["w"]),
-                      p(s["u"]), p(s_in), p(s["dy"]), p(s["dstate"]), p(self.gr), p(self.gk), p(self.gv), p(self.gw),
-                      p(self.gu), p(self.gstate_in), p(self.ws), self.ws.numel())
+                      p(s["u"]), p(s_in), p(s["dy"]), p(g_out), p(self.gr), p(self.gk), p(self.gv), p(self.gw),
+                      p(self.gu), p(g_in), p(ws), ws.numel())
         assert st == 0, self.L.wkv_strerror(st)
+
+    def step(self):
+        """forward, then backward, of one segment"""
+        i = self.i
+        self.i += 1
+        s = self.sets[i % len(self.sets)]
+        self._forward(s, self.state[i % 2], self.state[(i + 1) % 2], self.ws)
+        self._backward(s, self.state[i % 2], self.gstate[i % 2], self.gstate[(i + 1) % 2], self.ws)
+
+    def step_cold(self):
+        """Cold-cache order: the backward call of the segment whose forward call ran two steps ago (its checkpoints
+        wait in the workspace this step's forward call then takes over), then this step's forward call.  Same calls,
+        same bytes per step; between a segment's forward and its backward lie two other calls' worth of traffic."""
+        torch = self.torch
+        if self.ws_cold is None:
+            self.ws_cold = torch.empty_like(self.ws)
+        i = self.i
+        self.i += 1
+        n = len(self.sets)
+        ws = (self.ws, self.ws_cold)[i % 2]
+        if i >= 2:
+            self._backward(self.sets[(i - 2) % n], self.state[i % 2], self.gstate[i % 2], self.gstate[(i + 1) % 2], ws)
+        self._forward(self.sets[i % n], self.state[i % 2], self.state[(i + 1) % 2], ws)
 
     def kernel_ids(self):
         return {"forward": (1, 10), "backward": (2, 11)}
@@ -203,7 +242,7 @@ class Runner4:
         return {"forward": (3,), "backward": (4,)}
 
 
-def capture_steps(runner, nsteps):
+def capture_steps(runner, nsteps, step=None):
     """`nsteps` consecutive steps (input rotation x state ping-pong) recorded into a HIP graph.
     The library allocates nothing and synchronises nothing in a call, so its launches
     record as they are.  Returns None when the capture fails."""
@@ -217,7 +256,7 @@ def capture_steps(runner, nsteps):
             with torch.cuda.graph(g, stream=side):
                 runner.stream = torch.cuda.current_stream().cuda_stream
                 for _ in range(nsteps):
-                    runner.step()
+                    (step or runner.step)()
         torch.cuda.current_stream().wait_stream(side)
         return g
     except Exception as e:            # noqa: BLE001 - any capture problem means plain launches
@@ -533,6 +572,73 @@ def bench_block(a):
                       "torch_elementwise_ms": round(layer_t, 4), "speedup": round(layer_t / layer_k, 3), "parts": res}))
 
 
+def measure(runner, step, a):
+    """Warm up, then time exactly a.steps calls of `step` twice (host clock between two device synchronisations; HIP
+    events on the launch stream with the queue primed).  Returns ms per step both ways and how the steps were launched."""
+    torch = runner.torch
+    period = 2 * a.rotate if a.rotate % 2 else a.rotate        # input rotation x state ping-pong
+    runner.i = 0
+    for _ in range(-(-max(a.warmup, 2) // period) * period if a.launch == "graph" else max(a.warmup, 2)):
+        step()
+    torch.cuda.synchronize()
+    # The K timed steps as few graph launches as possible: up to 128 steps are ONE graph; a longer run replays a
+    # body of 120 steps (whole rotation periods) K // 120 times, plus one more graph with what is left.  A graph
+    # launch costs the host (and the idle GPU) about 0.2 ms, so a short run (the 20-step default of an automated
+    # harness) would otherwise measure launch latencies rather than the kernels.
+    body = tail = None
+    body_steps = a.steps if a.steps <= 128 else 120
+    if a.launch == "graph" and body_steps > 0:
+        body = capture_steps(runner, body_steps, step)
+        if body is not None and a.steps % body_steps:
+            tail = capture_steps(runner, a.steps % body_steps, step)
+            if tail is None:
+                body = None
+    graph = body
+    if graph is not None:
+        graph.replay()                 # untimed: the first replay uploads the graph
+        if tail is not None:
+            tail.replay()
+        torch.cuda.synchronize()
+
+    def run_k_steps():
+        if graph is not None:
+            for _ in range(a.steps // body_steps):
+                graph.replay()
+            if tail is not None:
+                tail.replay()
+        else:
+            for _ in range(a.steps):
+                step()
+
+    if a.settle_ms > 0 and graph is not None:      # untimed: the first replays of a fresh graph are slower than the steady state
+        t_end = time.perf_counter() + a.settle_ms * 1e-3
+        while time.perf_counter() < t_end:
+            run_k_steps()
+            torch.cuda.synchronize()
+    # (1) the K steps between two device synchronisations, by the host's clock.  This includes the latency of the
+    # first launch (about 0.2 - 0.6 ms for a graph: the GPU idles until the launch arrives), which is a property
+    # of the host, not of the kernels, and weighs 10 % and more on a 20-step run.
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_k_steps()
+    torch.cuda.synchronize()
+    ms_step_host = (time.perf_counter() - t0) / a.steps * 1e3
+    # (2) the same K steps once more, between two HIP events on the launch stream, with untimed plain steps
+    # queued in front so that the GPU is still busy when the timed launches arrive: the events then bracket
+    # exactly the K steps' execution.  This is the figure reported as ms_per_step / value.
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(period):            # (a whole period, so that the replayed graphs meet the state they were captured in)
+        step()
+    ev0.record()
+    run_k_steps()
+    ev1.record()
+    torch.cuda.synchronize()
+    launch = ((f"hip graph of {body_steps} steps per replay" + (f" + one of {a.steps % body_steps}" if tail is not None else ""))
+              if graph is not None else "eager")
+    return {"ms_per_step": ev0.elapsed_time(ev1) / a.steps, "ms_per_step_host": ms_step_host, "launch": launch,
+            "settle_ms": a.settle_ms if graph is not None else 0.0}
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -556,67 +662,14 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-    period = 2 * a.rotate if a.rotate % 2 else a.rotate        # input rotation x state ping-pong
-    for _ in range(-(-max(a.warmup, 1) // period) * period if a.launch == "graph" else a.warmup):
-        runner.step()
-    torch.cuda.synchronize()
-    # The K timed steps as few graph launches as possible: up to 128 steps are ONE graph; a longer run replays a
-    # body of 120 steps (whole rotation periods) K // 120 times, plus one more graph with what is left.  A graph
-    # launch costs the host (and the idle GPU) about 0.2 ms, so a short run (the 20-step default of an automated
-    # harness) would otherwise measure launch latencies rather than the kernels.
-    body = tail = None
-    body_steps = a.steps if a.steps <= 128 else 120
-    if a.launch == "graph" and body_steps > 0:
-        body = capture_steps(runner, body_steps)
-        if body is not None and a.steps % body_steps:
-            tail = capture_steps(runner, a.steps % body_steps)
-            if tail is None:
-                body = None
-    graph = body
-    if graph is not None:
-        graph.replay()                 # untimed: the first replay uploads the graph
-        if tail is not None:
-            tail.replay()
-        torch.cuda.synchronize()
-    def run_k_steps():
-        if graph is not None:
-            for _ in range(a.steps // body_steps):
-                graph.replay()
-            if tail is not None:
-                tail.replay()
-        else:
-            for _ in range(a.steps):
-                runner.step()
-
-    if a.settle_ms > 0 and graph is not None:      # untimed: the first replays of a fresh graph are slower than the steady state
-        t_end = time.perf_counter() + a.settle_ms * 1e-3
-        while time.perf_counter() < t_end:
-            run_k_steps()
-            torch.cuda.synchronize()
-    # (1) the K steps between two device synchronisations, by the host's clock.  This includes the latency of the
-    # first launch (about 0.2 - 0.6 ms for a graph: the GPU idles until the launch arrives), which is a property
-    # of the host, not of the kernels, and weighs 10 % and more on a 20-step run.
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_k_steps()
-    torch.cuda.synchronize()
-    ms_step_host = (time.perf_counter() - t0) / a.steps * 1e3
-    # (2) the same K steps once more, between two HIP events on the launch stream, with two untimed plain steps
-    # queued in front so that the GPU is still busy when the timed launches arrive: the events then bracket
-    # exactly the K steps' execution.  This is the figure reported as ms_per_step / value.
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(2):
-        runner.step()
-    ev0.record()
-    run_k_steps()
-    ev1.record()
-    torch.cuda.synchronize()
-    ms_step = ev0.elapsed_time(ev1) / a.steps
-    tok_s = runner.tokens_per_step / (ms_step * 1e-3)
+    step = runner.step_cold if (a.cold and a.cfg != 2) else runner.step
+    m = measure(runner, step, a)
+    ms_step, ms_step_host, tok_s = m["ms_per_step"], m["ms_per_step_host"], runner.tokens_per_step / (m["ms_per_step"] * 1e-3)
 
     # per-kernel launch durations (HIP events around the kernel, on its stream)
     ksteps = min(a.steps, 20)
     kern = {}
+    runner.i = 0
     for phase, ids in runner.kernel_ids().items():
         for kid in ids:
             ms = time_kernel(runner, kid, ksteps)
@@ -639,14 +692,25 @@ def main():
            "value": tok_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": runner.dtype_name, "data": "synthetic",
-           "config": {"workload": runner.desc, "algo": a.algo, "segments": a.segments or "auto",
-                      "launch": (f"hip graph of {body_steps} steps per replay" + (f" + one of {a.steps % body_steps}" if tail is not None else ""))
-                                if graph is not None else "eager"},
-           "ms_per_step_host": ms_step_host, "untimed_settle_ms": a.settle_ms if graph is not None else 0.0,
+           "config": {"workload": runner.desc + (", cold-cache order (backward of the segment two steps back, then this step's forward)" if a.cold and a.cfg != 2 else ""),
+                      "algo": a.algo, "segments": a.segments or "auto", "launch": m["launch"]},
+           "ms_per_step_host": ms_step_host, "untimed_settle_ms": m["settle_ms"],
            "timing": "ms_per_step and value: HIP events on the launch stream around exactly the K steps, the queue "
-                     "primed with two untimed steps; ms_per_step_host: the same K steps between two device "
+                     "primed with untimed plain steps; ms_per_step_host: the same K steps between two device "
                      "synchronisations by the host clock (includes the latency of the first launch)",
            "roofline": roofline}
+    if not a.no_extras and a.cfg != 2 and not a.cold:
+        frac = lambda ms, r: r.bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        c = measure(runner, runner.step_cold, a)
+        out["cold"] = {"ms_per_step": c["ms_per_step"], "whole_step_frac": frac(c["ms_per_step"], runner),
+                       "order": "backward of the segment whose forward ran two steps ago, then this step's forward; two workspaces"}
+        if runner.version == 6 and not a.w_shift:
+            del runner
+            torch.cuda.empty_cache()
+            slow = Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, -5.0, a.io_dtype)
+            sd = measure(slow, slow.step, a)
+            out["slow_decay"] = {"ms_per_step": sd["ms_per_step"], "whole_step_frac": frac(sd["ms_per_step"], slow),
+                                 "raw_decay_shift": -5.0}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(a.cfg, a.cpu_heads)
     print(json.dumps(out))

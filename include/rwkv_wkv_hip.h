@@ -78,6 +78,9 @@ int wkv_init(void);
  * forward call and its backward call (only the state checkpoints pass between the two, and those do not depend
  * on it). */
 #define WKV_TUNE_SEGMENTS 1
+/* WKV_TUNE_PIECE_STEPS: the summary pass of the time split cuts every segment into pieces of this many 64-token
+ * steps (one workgroup and one 16 KiB summary per piece); 0 = choose from the shape (default).  Same rules as above. */
+#define WKV_TUNE_PIECE_STEPS 2
 int wkv_tune(int key, int value);
 
 /* Timing hook for benchmarks (no counterpart in the reference).

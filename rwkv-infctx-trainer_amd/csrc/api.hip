@@ -149,6 +149,11 @@ int wkv_tune(int key, int value) {
         chunked::forced_segments() = value;
         return WKV_OK;
     }
+    if (key == WKV_TUNE_PIECE_STEPS) {
+        if (value < 0) return WKV_ERR_DIMS;
+        chunked::forced_piece_steps() = value;
+        return WKV_OK;
+    }
     return WKV_ERR_DIMS;
 }
 

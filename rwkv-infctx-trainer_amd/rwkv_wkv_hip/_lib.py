@@ -18,6 +18,7 @@ CHECKPOINTS_VALID = 2
 W_BF16 = 4          # WKV6, chunked algorithm: w and gw are bf16
 ALGO_AUTO, ALGO_RECURRENT, ALGO_CHUNKED = 0, 1, 2
 TUNE_SEGMENTS = 1
+TUNE_PIECE_STEPS = 2
 
 _P = c_void_p
 _I = c_int

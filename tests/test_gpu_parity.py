@@ -387,6 +387,45 @@ def test_chunked_time_segments(version, nseg, T):
     compare(got, ref, 2e-2, f"segments v{version}/n{nseg}/T{T}")
 
 
+def _slow_decay_case(kind, T):
+    """cfg3 data with the raw decay moved so that the summary passes of the time split cannot stop early.
+    RWKV-v6 initialises time_decay in [-6, -1] (decay 0.9975 .. 0.69 per token), the training case; the benchmark
+    distribution N(-1, 0.5) forgets within about a hundred tokens."""
+    from rwkv_wkv_hip import configs
+    wl = configs.make(3, B=1, T=T, C=256, H=4, dtype=torch.bfloat16)
+    w = wl.tensors["w"]
+    if kind == "all":                   # every head keeps its state across whole segments: no piece stops
+        w -= 5.0
+    elif kind == "half":                # heads 0, 1 slow, heads 2, 3 fast: neighbouring pieces report 0 and non-zero decays
+        w[:, :, :128] -= 5.0
+    elif kind == "turns":               # head 1 turns slow in the middle of a segment, head 2 turns fast there;
+        w[:, T // 4 + 96:, 64:128] -= 5.0       # single channels of head 3 stay slow while the others forget
+        w[:, :T // 4 + 96, 128:192] -= 5.0
+        w[:, :, 192:200] -= 6.0
+    return wl
+
+
+@pytest.mark.parametrize("kind", ["all", "half", "turns"])
+@pytest.mark.parametrize("nseg,pps", [(2, 0), (4, 0), (2, 8), (4, 3)])
+def test_chunked_time_segments_slow_decay(kind, nseg, pps):
+    """The time split with decays that do not forget inside a piece: the summary passes walk their pieces to the end
+    (no early exit), heads that stop and heads that do not sit side by side, and the chaining of the summaries in the
+    main kernels' prologues runs over every piece.  pps = steps per piece (0: the planner's choice, 2-step pieces
+    at this size; 8 and 3: pieces of several steps, ragged ones included).  All eight outputs against the oracle."""
+    from rwkv_wkv_hip import _lib
+    L = _lib.lib()
+    T = 2048
+    wl = _slow_decay_case(kind, T)
+    print(f"case slow decay {kind} nseg={nseg} pps={pps}", flush=True)
+    assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg) == 0 and L.wkv_tune(_lib.TUNE_PIECE_STEPS, pps) == 0
+    try:
+        got = run_gpu56(6, wl, algo="chunked")
+    finally:
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, 0) == 0 and L.wkv_tune(_lib.TUNE_PIECE_STEPS, 0) == 0
+    ref = run_oracle56(6, wl)
+    compare(got, ref, 2e-2, f"slow decay {kind}/n{nseg}/p{pps}")       # bf16 I/O: rtol 2e-2, floor 2e-2 rms
+
+
 @pytest.mark.parametrize("nseg,T", [(1, 200), (3, 1000)])
 def test_chunked_v6_takes_bf16_decay(nseg, T):
     """The raw decay handed over in bf16 (what a mixed-precision TimeMix produces and the reference widens with
