@@ -64,10 +64,11 @@ typedef enum { WKV_F32 = 0, WKV_BF16 = 1, WKV_F16 = 2 } wkv_dtype;
 const char *wkv_strerror(int status);
 int wkv_abi_version(void);
 
-/* One-time set-up of the loaded kernels on the current process (raises the LDS limit of the blocked kernels; no
- * counterpart in the reference, whose extension is configured when torch builds it, RWKV-v5/src/module/TimeMix.py:
- * 229-252).  The operators do it themselves on their first call; call it once beforehand when that first call
- * would fall inside a HIP stream capture.  Needs a GPU; returns WKV_ERR_LAUNCH without one. */
+/* One-time set-up of the loaded kernels (raises the LDS limit of the blocked kernels, once per process; looks up
+ * the address of wkv6_forward_noalloc's scratch array on the CURRENT device; no counterpart in the reference, whose
+ * extension is configured when torch builds it, RWKV-v5/src/module/TimeMix.py:229-252).  The operators do it
+ * themselves on their first call; call it beforehand, once per device with that device current, when that first
+ * call would fall inside a HIP stream capture.  Needs a GPU; returns WKV_ERR_LAUNCH without one. */
 int wkv_init(void);
 
 /* Tuning knobs (no counterpart in the reference).  WKV_TUNE_SEGMENTS: number of
@@ -111,7 +112,11 @@ int wkv_profile_end(float *ms, int capacity);
  * checkpoints there.  Passing that same buffer, sized by
  * wkv6_backward_workspace() (>= the forward size), to backward together with
  * WKV_CHECKPOINTS_VALID saves backward one sweep over k, v, w. */
-/* state_out must not overlap state_in (WKV_ERR_ALIAS); the same holds for wkv5_forward. */
+/* state_out == state_in (the state updated in place) is accepted by the per-token algorithm and by the chunked one
+ * whenever the plan cuts no sequence of the shape into time segments (B*H at least the number of compute units, or
+ * WKV_TUNE_SEGMENTS 1); where it does (short batches, e.g. the 7B shape with B = 1), and for buffers that overlap
+ * without being the same, the call returns WKV_ERR_ALIAS and the caller keeps two state buffers and alternates.
+ * The same holds for wkv5_forward and wkv6_forward_noalloc. */
 size_t wkv6_forward_workspace(int B, int T, int C, int H, int dtype, int algo);
 int wkv6_forward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
                  const void *r, const void *k, const void *v, const void *w, const float *u,

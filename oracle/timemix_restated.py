@@ -1,4 +1,4 @@
-"""Test-only restatement of the reference's TimeMix forward passes around the WKV
+"""Test infrastructure (only tests may use it): restatement of the reference's TimeMix forward passes around the WKV
 operator (RWKV-v5/src/module/TimeMix.py:286-366, RWKV-v6/src/module/TimeMix.py:253-351),
 with the operator injected, so that the same module can run on the CPU oracle
 (the reference's pure path) and on the HIP operators (its CUDA path)."""

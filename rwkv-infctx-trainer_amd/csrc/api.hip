@@ -35,6 +35,17 @@ int pick_algo56(int algo, int T, int dtype, unsigned flags) {
     return WKV_ERR_ALGO;
 }
 
+// state_out == state_in (the state updated in place, as a serving loop does) is fine whenever every workgroup reads
+// the state of its (batch, head) pair before it writes it: the per-token kernels, and the blocked ones as long as
+// no sequence is cut into time segments (then the workgroups of the later segments read state_in while the one of
+// the last segment writes state_out).  Buffers that overlap without being the same never are.
+static int check_state_alias(const float *state_in, const float *state_out, int B, int H, bool time_split) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(state_in), b0 = reinterpret_cast<uintptr_t>(state_out);
+    const size_t bytes = (size_t)B * H * HEAD * HEAD * sizeof(float);
+    if (!(a0 < b0 + bytes && b0 < a0 + bytes)) return WKV_OK;
+    return (a0 == b0 && !time_split) ? WKV_OK : WKV_ERR_ALIAS;
+}
+
 int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
               const void *r, const void *k, const void *v, const void *w, const float *u, const float *state_in,
               void *y, float *state_out, void *workspace, size_t workspace_bytes) {
@@ -44,13 +55,10 @@ int forward56(bool per_token, void *stream, int B, int T, int C, int H, int dtyp
     for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
                           (const void *)state_out})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
-    {
-        const uintptr_t a0 = reinterpret_cast<uintptr_t>(state_in), b0 = reinterpret_cast<uintptr_t>(state_out);
-        const size_t bytes = (size_t)B * H * HEAD * HEAD * sizeof(float);
-        if (a0 < b0 + bytes && b0 < a0 + bytes) return WKV_ERR_ALIAS;
-    }
     const int a = pick_algo56(algo, T, dtype, flags);
     if (a < 0) return a;
+    st = check_state_alias(state_in, state_out, B, H, a == WKV_ALGO_CHUNKED && chunked::splits_time(B * H, T));
+    if (st) return st;
     const bool w16 = (flags & WKV_W_BF16) != 0;
     if (w16 && (!per_token || a != WKV_ALGO_CHUNKED)) return WKV_ERR_ALGO;
     if (a == WKV_ALGO_CHUNKED) {
@@ -134,14 +142,17 @@ const char *wkv_strerror(int status) {
         case WKV_ERR_WORKSPACE: return "workspace too small";
         case WKV_ERR_LAUNCH: return "HIP launch failed";
         case WKV_ERR_ALGO: return "algorithm not available for this shape/dtype";
-        case WKV_ERR_ALIAS: return "state_out overlaps state_in";
+        case WKV_ERR_ALIAS: return "state_out overlaps state_in (in place is possible only where no sequence is cut into time segments)";
         default: return "unknown status";
     }
 }
 
 int wkv_abi_version(void) { return 2; }
 
-int wkv_init(void) { return chunked::init_kernels() == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH; }
+int wkv_init(void) {
+    if (chunked::init_kernels() != hipSuccess) return WKV_ERR_LAUNCH;
+    return chunked::init_static_scratch() == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;      // (for the current device)
+}
 
 int wkv_tune(int key, int value) {
     if (key == WKV_TUNE_SEGMENTS) {
@@ -215,12 +226,9 @@ int wkv6_forward_noalloc(void *stream, int B, int T, int C, int H, int dtype, un
     for (const void *p : {r, k, v, (const void *)w, (const void *)u, (const void *)state_in, (const void *)y,
                           (const void *)state_out})
         if (!aligned16(p)) return WKV_ERR_ALIGN;
-    {
-        const uintptr_t a0 = reinterpret_cast<uintptr_t>(state_in), b0 = reinterpret_cast<uintptr_t>(state_out);
-        const size_t bytes = (size_t)B * H * HEAD * HEAD * sizeof(float);
-        if (a0 < b0 + bytes && b0 < a0 + bytes) return WKV_ERR_ALIAS;
-    }
     if (pick_algo56(WKV_ALGO_CHUNKED, T, dtype, flags) != WKV_ALGO_CHUNKED) return WKV_ERR_ALGO;
+    st = check_state_alias(state_in, state_out, B, H, chunked::splits_time(B * H, T));
+    if (st) return st;
     hipError_t e = chunked::forward_static_launch((hipStream_t)stream, true, (flags & WKV_W_BF16) != 0, B, T, C, H, r, k, v, w,
                                                   u, state_in, y, state_out, (flags & WKV_FLOOR_DECAY) ? 1 : 0);
     if (e == hipErrorOutOfMemory) return WKV_ERR_WORKSPACE;

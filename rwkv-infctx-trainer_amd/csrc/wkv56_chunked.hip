@@ -1494,6 +1494,8 @@ static Layout layout(int B, int Tlen, int C, int H, const GroupPlan &gp) {
     L.total = L.sums + round256(2 * (size_t)B * (gp.b.nseg + 1) * C * sizeof(float));
     return L;
 }
+// true when the plan in force cuts some sequence of this shape into time segments
+bool splits_time(int BH, int Tlen) { return plan_groups(BH, Tlen).b.nseg > 1; }
 size_t forward_workspace(int B, int Tlen, int H) { return layout(B, Tlen, H * HEAD, H, plan_groups(B * H, Tlen)).forward_total; }
 size_t backward_workspace(int B, int Tlen, int C, int H) { return layout(B, Tlen, C, H, plan_groups(B * H, Tlen)).total; }
 

@@ -28,6 +28,12 @@ static hipError_t static_scratch_address(void **out) {
     *out = p;
     return hipSuccess;
 }
+// what wkv_init() does for this entry point: the array's address on the current device, so that the first call has
+// no set-up left to do (a first call inside a stream capture)
+hipError_t init_static_scratch() {
+    void *p = nullptr;
+    return static_scratch_address(&p);
+}
 // returns hipErrorOutOfMemory when the plan's summaries do not fit the array
 hipError_t forward_static_launch(hipStream_t s, bool per_token, bool w16, int B, int Tlen, int C, int H, const void *r, const void *k,
                                  const void *v, const void *w, const float *u, const float *s_in, void *y, float *s_out,

@@ -81,33 +81,91 @@ class RecomputeCache:
     RWKV-v5/src/model.py:674-683) the operator's forward runs twice per layer and segment: once without autograd
     while the model runs forward, once more when backward recomputes the block.  With a cache installed
     (``with recompute_cache(): ...`` around the training step) the first run keeps its outputs and its state
-    checkpoints, and the recomputation, which replays the blocks in reverse order, takes them over instead of
-    running the kernels again: one forward pass of the operator less per layer and segment, paid for with y, the new
-    state and the checkpoints (about 6 bytes per token and channel) held from forward to backward.
+    checkpoints, and the recomputation takes them over instead of running the kernels again: one forward pass of the
+    operator less per layer and segment, paid for with y, the new state and the checkpoints (about 6 bytes per token
+    and channel) held from forward to backward.
 
-    Matching is by order (last kept, first reused) and by signature (operator, shape, dtypes): it relies on the
-    recomputation replaying exactly the calls of the first run, as activation checkpointing does.  Forward runs
-    that are never recomputed (validation, generation) must stay outside the ``with`` block."""
+    Which kept run a call with autograd on may take over:
 
-    def __init__(self, max_entries: int = 4096):
-        self.stack, self.max_entries = [], max_entries
+    * keyed (recommended): the caller names each call, ``with call_key((layer, segment)): ...`` around the block's
+      forward.  A kept run is taken over only by a call with the same key and signature (operator, shape, dtypes);
+      any other call runs the kernels.  This is safe for every pattern, including the reference's outer per-segment
+      checkpoint (RWKV-v5/src/model.py:1248: segments 0..S-2 run without autograd, the last one with) and nested
+      checkpoints.
+    * unkeyed: last kept, first taken over, by signature.  This is what plain activation checkpointing of a stack of
+      equal layers does (the recomputation replays the blocks in reverse order) and nothing else: a call with
+      autograd on that is not a recomputation would take over another call's results.  That is why every take-over
+      is verified: 1024 elements spread over r, kept on the device from the first run, are compared with the
+      recomputation's r by a few asynchronous device operations, and ``check()`` (called on leaving the ``with`` block;
+      one synchronisation per step) raises if any take-over met different inputs.  The step's gradients are then
+      wrong and must be discarded; switch to keys.
 
-    def push(self, sig, payload):
-        if len(self.stack) >= self.max_entries:
-            self.stack.pop(0)
-        self.stack.append((sig, payload))
+    Kept runs that are never taken over (forward-only work inside the block, segments outside the BPTT range) stay
+    until the ``with`` block is left; ``max_bytes`` bounds what they hold (oldest dropped first).  Under nested
+    checkpoints an inner recomputation runs without autograd again and keeps its run a second time: harmless, the
+    copy is dropped on leaving."""
 
-    def pop(self, sig):
-        if self.stack and self.stack[-1][0] == sig:
-            return self.stack.pop()[1]
-        return None
+    SAMPLE = 1024
+
+    def __init__(self, max_entries: int = 4096, max_bytes: int = 16 << 30, verify: bool = True):
+        self.entries, self.max_entries, self.max_bytes, self.verify = [], max_entries, max_bytes, verify
+        self.bytes, self.bad = 0, None
+
+    @classmethod
+    def _sample(cls, r):
+        flat = r.reshape(-1)
+        step = max(flat.numel() // cls.SAMPLE, 1)
+        return flat[::step][:cls.SAMPLE].clone()
+
+    @staticmethod
+    def _nbytes(payload):
+        return sum(t.numel() * t.element_size() for t in payload if torch.is_tensor(t))
+
+    def push(self, key, sig, r, payload):
+        n = self._nbytes(payload)
+        while self.entries and (len(self.entries) >= self.max_entries or self.bytes + n > self.max_bytes):
+            self.bytes -= self.entries.pop(0)[4]
+        self.entries.append((key, sig, self._sample(r) if self.verify else None, payload, n))
+        self.bytes += n
+
+    def pop(self, key, sig, r):
+        hit = None
+        if key is None:         # unkeyed: the most recent kept run, if it is unkeyed too and has this signature
+            if self.entries and self.entries[-1][0] is None and self.entries[-1][1] == sig:
+                hit = self.entries.pop()
+        else:
+            for i in range(len(self.entries) - 1, -1, -1):
+                if self.entries[i][0] == key and self.entries[i][1] == sig:
+                    hit = self.entries.pop(i)
+                    break
+        if hit is None:
+            return None
+        self.bytes -= hit[4]
+        if hit[2] is not None:      # asynchronous: no host synchronisation here
+            differs = (hit[2] != self._sample(r)).any()
+            self.bad = differs if self.bad is None else (self.bad | differs)
+        return hit[3]
+
+    def check(self):
+        """Raises if a take-over since the last check met inputs that differ from the kept run's (synchronises)."""
+        bad, self.bad = self.bad, None
+        if bad is not None and bool(bad.item()):
+            raise WKVError("recompute cache: a kept forward run was taken over by a call with different inputs (a call "
+                           "with autograd on that was not the recomputation of that run); the gradients of this step "
+                           "are wrong.  Name the calls with call_key() or keep such calls outside recompute_cache()")
+
+    def clear(self):
+        self.entries.clear()
+        self.bytes = 0
 
 
 _cache = None
+_key = None
 
 
 class recompute_cache:
-    """Context manager that installs a ``RecomputeCache`` for the operators called inside it."""
+    """Context manager that installs a ``RecomputeCache`` for the operators called inside it; on leaving, the
+    take-overs are verified (``RecomputeCache.check``) and what is still kept is dropped."""
 
     def __init__(self, cache: RecomputeCache = None):
         self.cache = cache or RecomputeCache()
@@ -117,10 +175,33 @@ class recompute_cache:
         self.prev, _cache = _cache, self.cache
         return self.cache
 
-    def __exit__(self, *exc):
+    def __exit__(self, exc_type, *exc):
         global _cache
         _cache = self.prev
-        self.cache.stack.clear()
+        self.cache.clear()
+        if exc_type is None:
+            self.cache.check()
+        else:
+            self.cache.bad = None
+        return False
+
+
+class call_key:
+    """Names the operator calls made inside it for the recompute cache (any hashable: e.g. (layer, segment)).  The
+    same key must be in force when the block's forward is recomputed, which it is when the ``with`` sits inside the
+    checkpointed function."""
+
+    def __init__(self, key):
+        self.key = key
+
+    def __enter__(self):
+        global _key
+        self.prev, _key = _key, self.key
+        return self
+
+    def __exit__(self, *exc):
+        global _key
+        _key = self.prev
         return False
 
 
@@ -129,9 +210,9 @@ def _forward56_cached(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad, ou
     cache = _cache
     if cache is None:
         return _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad, out_state)
-    sig = (version, B, T, C, H, r.dtype, w32.dtype, tuple(w32.shape))
+    sig = (version, B, T, C, H, r.dtype, w32.dtype, tuple(w32.shape), out_state is not None)
     if need_grad:
-        hit = cache.pop(sig)
+        hit = cache.pop(_key, sig, r)
         if hit is not None:          # the recomputation of a forward run that kept its results
             y, new_state, ws, algo = hit
             if out_state is not None:
@@ -141,7 +222,7 @@ def _forward56_cached(version, B, T, C, H, r, k, v, w32, u32, s32, need_grad, ou
             return y, new_state, ws, algo
         return _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, True, out_state)
     y, new_state, ws, algo = _forward56(version, B, T, C, H, r, k, v, w32, u32, s32, True, out_state)    # keep checkpoints
-    cache.push(sig, (y, new_state.clone() if out_state is not None else new_state, ws, algo))
+    cache.push(_key, sig, r, (y, new_state.clone() if out_state is not None else new_state, ws, algo))
     return y, new_state, ws, algo
 
 

@@ -8,7 +8,7 @@ import torch
 
 from oracle import blocks as OB
 from oracle import wkv56 as O
-from tests.timemix_restated import ChannelMix5, ChannelMix6, TimeMix5, TimeMix6
+from oracle.timemix_restated import ChannelMix5, ChannelMix6, TimeMix5, TimeMix6
 from tests.util import assert_close
 
 pytestmark = pytest.mark.gpu

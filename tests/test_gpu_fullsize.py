@@ -198,3 +198,40 @@ def test_long_context_chain_7b_shape():
         if seg % 16 == 0:
             print(f"segment {seg}: drift {drift:.2e}", flush=True)
     print("worst max-error / rms per tensor over the chain:", {k: f"{v:.2e}" for k, v in worst.items()}, flush=True)
+
+
+def test_full_shape_cumsum_decay_helper():
+    """The helper at the shape `bench.py --helper` times (raw decay of cfg3: B8 T4096 C2560, chunk length 128, where
+    the chunk's log decays stay in registers): every log-space table of every element against the oracle, one batch
+    row at a time, and the exponentiated tables and fp64 re-centred factors of the first and last row."""
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import configs
+    wl = configs.make(3)
+    B, T, C, H, chunk = wl.B, wl.T, wl.C, wl.H, 128
+    print(f"case helper B{B} T{T} C{C} chunk {chunk}", flush=True)
+    raw = wl.tensors["w"].clone()
+    raw[0, 9, 5] = 3.0                      # below the floor
+    raw[B - 1, T - 1, C - 1] = 2.0
+    out = W.cumsum_decay(raw.to(DEV), chunk, factors=True, precision=64)
+    torch.cuda.synchronize()
+    back = lambda x: x.reshape(1, H, T, 64).transpose(1, 2).reshape(T, C)
+    lg = lambda x: x.double().log().float()
+    for b in range(B):
+        w = O.decay_from_raw(raw[b:b + 1]).view(1, T, H, 64).transpose(1, 2)
+        tab = O.cumsum_decay(w, chunk, 64)
+        assert_close(out["log_w"][b], back(tab.log_w), 1e-5, f"log_w row {b}")
+        assert_close(out["incl"][b], back(tab.incl), 1e-5, f"incl row {b}")
+        assert_close(out["inter"][b], back(tab.inter_log), 1e-5, f"inter row {b}")
+        assert_close(out["intra"][b], back(tab.intra_log), 1e-5, f"intra row {b}")
+        cs = tab.chunk_log[..., 0, :].transpose(1, 2).reshape(T // chunk, C)
+        assert_close(out["chunk_sum"][b], cs, 1e-5, f"chunk_sum row {b}")
+        if b in (0, B - 1):
+            # (exponentials below the smallest normal fp32 come back as 0 from the GPU: absolute floor 1e-37; the
+            # exponents are fp32 sums of up to 128 terms summed in another order by torch: 2e-4 relative)
+            near = lambda a, r, n: torch.testing.assert_close(a.cpu(), r, rtol=2e-4, atol=1e-37, msg=lambda m: f"{n}: {m}")
+            near(out["ws_exp"][b], cs.exp(), "ws_exp")
+            near(out["inter_exp"][b], back(tab.inter_log).exp(), "inter_exp")
+            near(out["intra_exp"][b], back(tab.intra_log).exp(), "intra_exp")
+            assert_close(lg(out["r_decay"][b].cpu()), lg(back(tab.r_decay)), 1e-5, f"log r_decay row {b}")
+            assert_close(lg(out["k_inv_decay"][b].cpu()), lg(back(tab.k_inv_decay)), 1e-5, f"log k_inv_decay row {b}")
+    assert out["log_w"][0, 9, 5].item() == pytest.approx(-5.298317, abs=1e-5)

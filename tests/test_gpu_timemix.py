@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import wkv56 as O
-from tests.timemix_restated import TimeMix5, TimeMix6
+from oracle.timemix_restated import TimeMix5, TimeMix6
 from tests.util import assert_close
 
 pytestmark = pytest.mark.gpu

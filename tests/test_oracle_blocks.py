@@ -81,7 +81,7 @@ def test_l2wrap_backward_against_a_row_loop():
 
 def test_channelmix_forms_agree():
     import torch.nn as nn
-    from tests.timemix_restated import ChannelMix5, ChannelMix6
+    from oracle.timemix_restated import ChannelMix5, ChannelMix6
     C = 16
     m5, m6 = ChannelMix5(C, 4 * C, seed=1).double(), ChannelMix6(C, 4 * C, seed=1).double()
     with torch.no_grad():       # same layer expressed in both parametrisations

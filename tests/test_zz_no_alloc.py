@@ -25,16 +25,20 @@ def _both(B, T, H, seed):
                         p(g["w"]), p(g["u"]), p(g["state"]), p(y0), p(s0), p(ws), ws.numel())
     assert st == 0, L.wkv_strerror(st)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # device memory as the driver counts it (hipMemGetInfo): an allocation inside the library would show here,
+    # whichever allocator made it; torch's own counter beside it
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     st = L.wkv6_forward_noalloc(stream, B, T, C, H, _lib.WKV_BF16, flags, p(g["r"]), p(g["k"]), p(g["v"]), p(g["w"]),
                                 p(g["u"]), p(g["state"]), p(y1), p(s1))
     assert st == 0, L.wkv_strerror(st)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_allocated() == before and torch.cuda.mem_get_info()[0] == free_before
     return (y0, s0), (y1, s1)
 
 
 def test_noalloc_forward_matches_workspace_forward_twice():
+    from rwkv_wkv_hip import _lib
+    assert _lib.lib().wkv_init() == 0          # (also looks up the scratch array's address: nothing left for the first call)
     for B, T, H, seed in ((1, 2048, 4, 11), (1, 1024, 2, 12)):        # both are cut into several time segments
         print(f"case noalloc B{B} T{T} H{H}", flush=True)
         (y0, s0), (y1, s1) = _both(B, T, H, seed)
@@ -44,13 +48,65 @@ def test_noalloc_forward_matches_workspace_forward_twice():
 
 
 def test_noalloc_forward_rejects_what_does_not_fit():
-    from rwkv_wkv_hip import _lib
+    """A plan whose piece summaries exceed the 16 MiB array is refused before anything is launched.  The plan is
+    forced (8 segments for 128 (batch, head) pairs: 128 x 8 summaries of 16.6 KB at least), and every pointer is a
+    real buffer of the right size, so that the call would be harmless even if the check were missing."""
+    from rwkv_wkv_hip import _lib, configs
     L = _lib.lib()
-    one = ctypes.c_void_p(4096)         # never dereferenced: the size check comes before any launch
-    two = ctypes.c_void_p(1 << 30)
-    st = L.wkv6_forward_noalloc(None, 8, 4096, 2560, 40, _lib.WKV_BF16, _lib.FLOOR_DECAY, one, one, one, one, one, one,
-                                one, two)
+    B, T, H = 2, 1024, 64
+    C = H * 64
+    wl = configs.make(3, seed=13, B=B, T=T, C=C, H=H, dtype=torch.bfloat16)
+    g = {n: x.cuda().contiguous() for n, x in wl.tensors.items()}
+    y, s = torch.empty_like(g["r"]), torch.empty_like(g["state"])
+    p = lambda t: t.data_ptr()
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.wkv_tune(_lib.TUNE_SEGMENTS, 8) == 0
+    try:
+        st = L.wkv6_forward_noalloc(stream, B, T, C, H, _lib.WKV_BF16, _lib.FLOOR_DECAY, p(g["r"]), p(g["k"]), p(g["v"]),
+                                    p(g["w"]), p(g["u"]), p(g["state"]), p(y), p(s))
+    finally:
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, 0) == 0
+    torch.cuda.synchronize()
     assert st == -5 and b"workspace" in L.wkv_strerror(st)
     # fp32 streams do not take the blocked algorithm
-    st = L.wkv6_forward_noalloc(None, 1, 128, 64, 1, _lib.WKV_F32, _lib.FLOOR_DECAY, one, one, one, one, one, one, one, two)
+    f = {n: (x.float() if x.dtype == torch.bfloat16 else x) for n, x in g.items()}
+    yf = torch.empty_like(f["r"])
+    st = L.wkv6_forward_noalloc(stream, B, T, C, H, _lib.WKV_F32, _lib.FLOOR_DECAY, p(f["r"]), p(f["k"]), p(f["v"]), p(f["w"]),
+                                p(f["u"]), p(f["state"]), p(yf), p(s))
     assert st == -7
+
+
+def test_state_in_place_where_no_sequence_is_cut():
+    """state_out == state_in: accepted by the per-token kernels and by the blocked ones when the plan cuts nothing in
+    time (same results as with two buffers), refused (WKV_ERR_ALIAS) when it does, and always for partial overlap."""
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    B, T, H = 1, 512, 2
+    C = H * 64
+    wl = configs.make(3, seed=14, B=B, T=T, C=C, H=H, dtype=torch.bfloat16)
+    g = {n: x.cuda().contiguous() for n, x in wl.tensors.items()}
+    p = lambda t: t.data_ptr()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fwd(algo, s_in, s_out, nseg):
+        y = torch.empty_like(g["r"])
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg) == 0
+        try:
+            st = L.wkv6_forward(stream, B, T, C, H, _lib.WKV_BF16, _lib.FLOOR_DECAY, algo, p(g["r"]), p(g["k"]), p(g["v"]),
+                                p(g["w"]), p(g["u"]), p(s_in), p(y), p(s_out), None, 0)
+        finally:
+            assert L.wkv_tune(_lib.TUNE_SEGMENTS, 0) == 0
+        torch.cuda.synchronize()
+        return st, y
+    for algo in (_lib.ALGO_RECURRENT, _lib.ALGO_CHUNKED):
+        two = torch.empty_like(g["state"])
+        st, y2 = fwd(algo, g["state"], two, 1)
+        assert st == 0
+        one = g["state"].clone()
+        st, y1 = fwd(algo, one, one, 1)
+        assert st == 0, L.wkv_strerror(st)
+        assert torch.equal(y1, y2) and torch.equal(one, two)
+    one = g["state"].clone()
+    assert fwd(_lib.ALGO_CHUNKED, one, one, 4)[0] == -8                 # cut in time: two buffers needed
+    big = torch.zeros(2 * g["state"].numel(), device="cuda")
+    assert fwd(_lib.ALGO_RECURRENT, big[:g["state"].numel()], big[64:64 + g["state"].numel()], 1)[0] == -8      # partial overlap
