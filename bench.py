@@ -55,10 +55,10 @@ def parse():
     ap.add_argument("--w-dtype", default="fp32", choices=["fp32", "bf16"],
                     help="WKV6 only: dtype of the raw decay tensor and its gradient (fp32 is what the workload is "
                          "defined with; bf16 is what a mixed-precision TimeMix hands over)")
-    ap.add_argument("--io-dtype", default="bf16", choices=["bf16", "fp16", "fp32"],
-                    help="WKV5/WKV6: dtype of r, k, v, dy and of y, gr, gk, gv (the workloads are defined in bf16; fp16 and "
-                         "fp32 run the per-token kernels, the reference binds all three, "
-                         "RWKV-v5/src/module/cuda/wkv5_op.cpp:84-129)")
+    ap.add_argument("--io-dtype", default=None, choices=["bf16", "fp16", "fp32"],
+                    help="dtype of r, k, v, dy and of y, gr, gk, gv.  Default: what the workload states (bf16 for WKV5/WKV6, "
+                         "fp32 for WKV4).  The reference binds all three for WKV5 (RWKV-v5/src/module/cuda/wkv5_op.cpp:84-129) "
+                         "and bf16 alone for WKV4 (RWKV-v4neo/cuda/wkv_op_bf16.cpp:45-51)")
     ap.add_argument("--helper", action="store_true",
                     help="time the cumulative-decay helper alone (all tables, chunk length 128) on the raw decay tensor of "
                          "--cfg 3 instead of the operators")
@@ -68,6 +68,9 @@ def parse():
     ap.add_argument("--block", action="store_true",
                     help="time one whole RWKV-v6 TimeMix + ChannelMix layer (cfg4 width, fwd+bwd): element-wise passes on the "
                          "HIP kernels against the same layer with torch element-wise ops around the same WKV operator")
+    ap.add_argument("--block-way", default="both", choices=["both", "kernels", "torch"],
+                    help="--block: time only the layer on the HIP element-wise kernels, only the one with torch element-wise "
+                         "ops, or both (for a profile of one of them alone)")
     ap.add_argument("--w-shift", type=float, default=0.0,
                     help="WKV6 only: added to the raw decay parameter (negative = slower decay; -5 makes every channel "
                          "remember for thousands of tokens, the worst case of the time-parallel split's summary passes)")
@@ -196,17 +199,23 @@ class Runner56:
 
 
 class Runner4:
-    """WKV4 forward+backward through the C ABI (cfg2)."""
+    """WKV4 forward+backward through the C ABI (cfg2; fp32 as the workload states it, or bf16 k/v/y/gradients, the only
+    dtype the reference's own kernel has, RWKV-v4neo/cuda/wkv_op_bf16.cpp:45-51)."""
 
-    def __init__(self, cfg, algo, rotate):
+    def __init__(self, cfg, algo, rotate, io_dtype="fp32"):
         import torch
         from rwkv_wkv_hip import _lib, configs
         self.torch, self._lib, self.L = torch, _lib, _lib.lib()
         dev = torch.device("cuda:0")
+        io = {"bf16": torch.bfloat16, "fp32": torch.float32}[io_dtype]
+        self.dt = {torch.float32: 0, torch.bfloat16: 1}[io]
         self.sets = []
         for i in range(rotate):
             wl = configs.make(cfg, seed=1000 + cfg + i)
-            self.sets.append({n: t.to(dev).contiguous() for n, t in wl.tensors.items()})
+            st = {n: t.to(dev).contiguous() for n, t in wl.tensors.items()}
+            for n in ("k", "v", "dy"):
+                st[n] = st[n].to(io)
+            self.sets.append(st)
         B, T, C = wl.B, wl.T, wl.C
         self.dims = (B, T, C)
         s0 = self.sets[0]
@@ -215,14 +224,15 @@ class Runner4:
         self.state = [s0["state"].clone(), torch.empty_like(s0["state"])]
         self.gstate = torch.empty_like(s0["state"])
         self.ckpt = torch.empty(self.L.wkv4_checkpoint_bytes(B, T, C), dtype=torch.uint8, device=dev)
-        self.ws = torch.empty(self.L.wkv4_backward_workspace(B, T, C, 0), dtype=torch.uint8, device=dev)
+        self.ws = torch.empty(self.L.wkv4_backward_workspace(B, T, C, self.dt), dtype=torch.uint8, device=dev)
         self.stream = torch.cuda.current_stream().cuda_stream
         self.i = 0
         self.tokens_per_step = B * T
         elems = B * T * C
-        self.bytes_step, self.bytes_fwd, self.bytes_bwd = 32 * elems, 12 * elems, 20 * elems
-        self.dtype_name = "f32"
-        self.desc = f"cfg{cfg}: WKV4 fwd+bwd B{B} T{T} C{C} fp32, (aa,bb,pp) state carried step to step"
+        eb = 4 if io == torch.float32 else 2
+        self.bytes_step, self.bytes_fwd, self.bytes_bwd = 8 * eb * elems, 3 * eb * elems, 5 * eb * elems
+        self.dtype_name = "f32" if io == torch.float32 else "bf16"
+        self.desc = f"cfg{cfg}: WKV4 fwd+bwd B{B} T{T} C{C} {io_dtype} k/v/dy, (aa,bb,pp) state fp32 carried step to step"
 
     def step(self):
         B, T, C = self.dims
@@ -230,10 +240,10 @@ class Runner4:
         s_in, s_out = self.state[self.i % 2], self.state[(self.i + 1) % 2]
         self.i += 1
         p = lambda t: t.data_ptr()
-        st = self.L.wkv4_forward(self.stream, B, T, C, 0, p(s["time_decay"]), p(s["time_first"]), p(s["k"]), p(s["v"]),
+        st = self.L.wkv4_forward(self.stream, B, T, C, self.dt, p(s["time_decay"]), p(s["time_first"]), p(s["k"]), p(s["v"]),
                                  p(s_in), p(self.y), p(s_out), p(self.ckpt))
         assert st == 0
-        st = self.L.wkv4_backward(self.stream, B, T, C, 0, p(s["time_decay"]), p(s["time_first"]), p(s["k"]), p(s["v"]),
+        st = self.L.wkv4_backward(self.stream, B, T, C, self.dt, p(s["time_decay"]), p(s["time_first"]), p(s["k"]), p(s["v"]),
                                   p(s_in), p(s["dy"]), None, p(self.gtd), p(self.gtf), p(self.gk), p(self.gv),
                                   p(self.gstate), p(self.ckpt), p(self.ws), self.ws.numel())
         assert st == 0
@@ -556,10 +566,18 @@ def bench_block(a):
         ev1.record()
         torch.cuda.synchronize()
         res[name] = round(ev0.elapsed_time(ev1) / n, 4)
-    timed("timemix_kernels_ms", lambda: K.timemix6_forward(tm, x, (shift, state))[0])
-    timed("timemix_torch_elementwise_ms", lambda: timemix_torch(tm, x, (shift, state))[0])
-    timed("channelmix_kernels_ms", lambda: K.channelmix6_forward(cm, x, shift)[0])
-    timed("channelmix_torch_elementwise_ms", lambda: channelmix_torch(cm, x, shift)[0])
+    if a.block_way in ("both", "kernels"):
+        timed("timemix_kernels_ms", lambda: K.timemix6_forward(tm, x, (shift, state))[0])
+        timed("channelmix_kernels_ms", lambda: K.channelmix6_forward(cm, x, shift)[0])
+    if a.block_way in ("both", "torch"):
+        timed("timemix_torch_elementwise_ms", lambda: timemix_torch(tm, x, (shift, state))[0])
+        timed("channelmix_torch_elementwise_ms", lambda: channelmix_torch(cm, x, shift)[0])
+    if a.block_way != "both":
+        way = "kernels" if a.block_way == "kernels" else "torch_elementwise"
+        print(json.dumps({"metric": f"RWKV-v6 layer (TimeMix + ChannelMix) fwd+bwd, B1 T4096 C4096 H64 bf16, {a.block_way} way only", "unit": "ms",
+                          "n_gpus": 1, "data": "synthetic", "dtype": "bf16", "higher_is_better": False,
+                          "value": round(res[f"timemix_{way}_ms"] + res[f"channelmix_{way}_ms"], 4), "parts": res}))
+        return
     with torch.no_grad():       # the two ways agree
         ya, yb = K.timemix6_forward(tm, x, (shift, state))[0].float(), timemix_torch(tm, x, (shift, state))[0].float()
         res["timemix_rel_diff"] = round(((ya - yb).norm() / yb.norm()).item(), 5)
@@ -653,7 +671,9 @@ def main():
         return bench_edges(a)
     if a.block:
         return bench_block(a)
-    runner = Runner4(a.cfg, a.algo, a.rotate) if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift, a.io_dtype)
+    if a.cfg == 2 and a.io_dtype == "fp16":
+        sys.exit("bench.py: --cfg 2 takes --io-dtype fp32 (the workload as stated, the default there) or bf16")
+    runner = Runner4(a.cfg, a.algo, a.rotate, a.io_dtype or "fp32") if a.cfg == 2 else Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, a.w_shift, a.io_dtype or "bf16")
     assert runner.L.wkv_tune(runner._lib.TUNE_SEGMENTS, a.segments) == 0
 
     if a.traffic_probe:
@@ -707,7 +727,7 @@ def main():
         if runner.version == 6 and not a.w_shift:
             del runner
             torch.cuda.empty_cache()
-            slow = Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, -5.0, a.io_dtype)
+            slow = Runner56(a.cfg, a.algo, a.rotate, a.w_dtype, -5.0, a.io_dtype or "bf16")
             sd = measure(slow, slow.step, a)
             out["slow_decay"] = {"ms_per_step": sd["ms_per_step"], "whole_step_frac": frac(sd["ms_per_step"], slow),
                                  "raw_decay_shift": -5.0}

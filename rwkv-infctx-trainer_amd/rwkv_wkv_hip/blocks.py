@@ -228,8 +228,11 @@ def timemix6_forward(self, x, last_state):
     xw, xk, xv, xr, xg = token_shift_mix(
         x, last_state[0], (self.time_maa_w, self.time_maa_k, self.time_maa_v, self.time_maa_r, self.time_maa_g), dyn=dyn)
     r, k, v, gate = self.receptance(xr), self.key(xk), self.value(xv), self.gate(xg)
-    w = self.time_decay + torch.tanh(xw @ self.time_decay_w1) @ self.time_decay_w2
-    y, new_state = WKV_6.apply(B, T, C, H, r, k, v, w.contiguous(), self.time_faaaa, last_state[1])
+    # w = time_decay + tanh(xw @ w1) @ w2 (TimeMix.py:280-281): the broadcast addition rides on the second matmul as
+    # its bias epilogue instead of being a pass of its own over (B,T,C)
+    lora = torch.tanh(xw.view(B * T, C) @ self.time_decay_w1)
+    w = torch.addmm(self.time_decay.reshape(C), lora, self.time_decay_w2).view(B, T, C)
+    y, new_state = WKV_6.apply(B, T, C, H, r, k, v, w, self.time_faaaa, last_state[1])
     y = ln_x_gate(y, gate, self.ln_x.weight, self.ln_x.bias, self.ln_x.eps, scale=1.0)
     return self.output(y), (x[:, -1], new_state)
 

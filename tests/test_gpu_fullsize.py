@@ -159,6 +159,35 @@ def test_full_shape_v4():
     assert_close(torch.cat([y1, y2], 1), y, 1e-4, "v4 chain y")
 
 
+def test_full_shape_v4_bf16():
+    """cfg2 at its full width in the reference kernel's own dtype (bf16 k, v, y and gradients,
+    RWKV-v4neo/cuda/wkv_op_bf16.cpp:45-51): B8 T4096 C4096 against the C oracle on the rounded inputs,
+    rtol 2e-2 (floor 2e-2 rms); the parameter gradients are sums over 32768 rounded terms per channel."""
+    import rwkv_wkv_hip as W
+    from rwkv_wkv_hip import configs
+    wl = configs.make(2, dtype=torch.bfloat16)
+    B, T, C = wl.B, wl.T, wl.C
+    print(f"case full cfg2: v4 B{B} T{T} C{C} bf16", flush=True)
+    cpu = wl.tensors
+    t = {n: x.to(DEV) for n, x in cpu.items()}
+    L = {n: t[n].clone().requires_grad_(True) for n in ("time_decay", "time_first", "k", "v", "state")}
+    y, s = W.wkv_op(L["time_decay"], L["time_first"], L["k"], L["v"], L["state"])
+    assert y.dtype == torch.bfloat16
+    torch.autograd.backward([y, s], [t["dy"], t["dstate"]])
+    torch.cuda.synchronize()
+    f32 = lambda x: x.float()
+    yr, sr = O4.forward(cpu["time_decay"], f32(cpu["time_first"]), f32(cpu["k"]), f32(cpu["v"]), cpu["state"])
+    ref = O4.backward(cpu["time_decay"], f32(cpu["time_first"]), f32(cpu["k"]), f32(cpu["v"]), cpu["state"], f32(cpu["dy"]),
+                      cpu["dstate"])
+    assert_close(y, yr, 2e-2, "v4 bf16 y")
+    und = lambda st: st[..., :2].float().cpu() * torch.exp(st[..., 2:3].float().cpu())
+    assert_close(und(s), und(sr), 1e-3, "v4 bf16 state")
+    assert_close(L["time_decay"].grad, ref[0], 2e-2, "v4 bf16 g_time_decay")
+    assert_close(L["time_first"].grad, ref[1], 2e-2, "v4 bf16 g_time_first")
+    assert_close(L["k"].grad, ref[2], 2e-2, "v4 bf16 gk")
+    assert_close(L["v"].grad, ref[3], 2e-2, "v4 bf16 gv")
+
+
 def test_long_context_chain_7b_shape():
     """cfg4: 64 consecutive 4096-token segments at B1 C4096 H64, fp32 state carried
     segment to segment on the GPU, forward + backward per segment.  All 64 heads are
