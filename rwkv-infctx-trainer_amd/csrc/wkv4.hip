@@ -76,19 +76,21 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
     if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
 
     // RING 16-token blocks of k, v per lane: one being consumed, the others in flight; indexed statically by unrolling
+    // (kept as they came: converting at the fetch would make every load wait for its data on the spot, and nothing
+    // would be in flight; the conversion happens where a value is used)
     constexpr int RING = 4;
-    float bk[RING][CK], bv[RING][CK];
-    auto fetch = [&](int t0, float (&kk)[CK], float (&vv)[CK]) {
+    T bk[RING][CK], bv[RING][CK];
+    auto fetch = [&](int t0, T (&kk)[CK], T (&vv)[CK]) {
         const T *kp = k + base + (size_t)t0 * C, *vp = v + base + (size_t)t0 * C;
         if (t0 + CK <= Tlen) {          // whole block inside the sequence: no per-token checks
 #pragma unroll
-            for (int i = 0; i < CK; i++, kp += C, vp += C) { kk[i] = to_float(*kp); vv[i] = to_float(*vp); }
+            for (int i = 0; i < CK; i++, kp += C, vp += C) { kk[i] = *kp; vv[i] = *vp; }
         } else {
 #pragma unroll
             for (int i = 0; i < CK; i++, kp += C, vp += C) {
                 const bool in = t0 + i < Tlen;
-                kk[i] = in ? to_float(*kp) : 0.f;
-                vv[i] = in ? to_float(*vp) : 0.f;
+                kk[i] = in ? *kp : T{};
+                vv[i] = in ? *vp : T{};
             }
         }
     };
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
                 for (int i = 0; i < CK; i++) {
                     if (decltype(full)::value || i < cnt) {
                         float iden, ec, hw, nm;
-                        const float yy = v4_step(s, w, u, bk[d][i], bv[d][i], iden, ec, hw, nm);
+                        const float yy = v4_step(s, w, u, to_float(bk[d][i]), to_float(bv[d][i]), iden, ec, hw, nm);
                         if (decltype(with_y)::value) { *yp = from_float<T>(yy); yp += C; }
                     }
                 }
@@ -156,21 +158,21 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
     const int nblk = (Tlen + CK - 1) / CK;
 
     // RB blocks of k, v, gy per lane: one being consumed, the others in flight
-    float bk[RB][CK], bv[RB][CK], bg[RB][CK];
-    auto fetch = [&](int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK]) {
+    T bk[RB][CK], bv[RB][CK], bg[RB][CK];        // (as they came; converted where they are used)
+    auto fetch = [&](int blk, T (&kk)[CK], T (&vv)[CK], T (&gg)[CK]) {
         const int t0 = blk * CK;
         const size_t o0 = base + (size_t)t0 * C;
         const T *kp = k + o0, *vp = v + o0, *gp_ = gy + o0;
         if (t0 + CK <= Tlen) {          // whole block inside the sequence: no per-token checks
 #pragma unroll
-            for (int i = 0; i < CK; i++, kp += C, vp += C, gp_ += C) { kk[i] = to_float(*kp); vv[i] = to_float(*vp); gg[i] = to_float(*gp_); }
+            for (int i = 0; i < CK; i++, kp += C, vp += C, gp_ += C) { kk[i] = *kp; vv[i] = *vp; gg[i] = *gp_; }
         } else {
 #pragma unroll
             for (int i = 0; i < CK; i++, kp += C, vp += C, gp_ += C) {
                 const bool in = t0 + i < Tlen;
-                kk[i] = in ? to_float(*kp) : 0.f;
-                vv[i] = in ? to_float(*vp) : 0.f;
-                gg[i] = in ? to_float(*gp_) : 0.f;
+                kk[i] = in ? *kp : T{};
+                vv[i] = in ? *vp : T{};
+                gg[i] = in ? *gp_ : T{};
             }
         }
     };
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
 #pragma unroll
         for (int d = 0; d < RB; d++)
             if (nblk - 1 - d >= 0) { fetch(nblk - 1 - d, bk[d], bv[d], bg[d]); bs[d] = load_ckpt(nblk - 1 - d); }
-        auto replay = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain s, V4Replay &out) {
+        auto replay = [&](auto full_tag, int blk, T (&kk)[CK], T (&vv)[CK], T (&gg)[CK], Chain s, V4Replay &out) {
             constexpr bool FULL = decltype(full_tag)::value;
             const int cnt = FULL ? CK : Tlen - blk * CK;
 #pragma unroll
@@ -194,9 +196,10 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
                 if (FULL || i < cnt) {
                     const float dp0 = s.dp, dq0 = s.dq;
                     float hw, iden, ec, nm;
-                    const float yy = v4_step(s, w, u, kk[i], vv[i], iden, ec, hw, nm);
-                    acc_w += gg[i] * (dp0 - dq0 * yy) * iden * hw;
-                    acc_u += gg[i] * (vv[i] - yy) * ec * iden;
+                    const float ki = to_float(kk[i]), vi = to_float(vv[i]), gi = to_float(gg[i]);
+                    const float yy = v4_step(s, w, u, ki, vi, iden, ec, hw, nm);
+                    acc_w += gi * (dp0 - dq0 * yy) * iden * hw;
+                    acc_u += gi * (vi - yy) * ec * iden;
                     out.ys[i][lane] = yy; out.iden[i][lane] = iden; out.ec[i][lane] = ec; out.neg_m[i][lane] = nm;
                 }
             }
@@ -206,7 +209,7 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
                 acc_w += (gp * s.dp + gq * s.dq) * __expf(s.o + go);
             }
         };
-        auto step = [&](int j, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], Chain &cs, V4Replay &out) {
+        auto step = [&](int j, T (&kk)[CK], T (&vv)[CK], T (&gg)[CK], Chain &cs, V4Replay &out) {
             const int blk = nblk - 1 - j;
             if (blk >= 0) {
                 if ((blk + 1) * CK <= Tlen) replay(std::true_type{}, blk, kk, vv, gg, cs, out);
@@ -232,7 +235,7 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
 #pragma unroll
         for (int d = 0; d < RB; d++)
             if (nblk - 1 - d >= 0) fetch(nblk - 1 - d, bk[d], bv[d], bg[d]);
-        auto walk = [&](auto full_tag, int blk, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], const V4Replay &in) {
+        auto walk = [&](auto full_tag, int blk, T (&kk)[CK], T (&vv)[CK], T (&gg)[CK], const V4Replay &in) {
             constexpr bool FULL = decltype(full_tag)::value;
             const int t0 = blk * CK, cnt = FULL ? CK : Tlen - t0;
             const size_t oe = base + (size_t)(t0 + CK - 1) * C;
@@ -241,20 +244,21 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
             for (int i = CK - 1; i >= 0; i--, gkp -= C, gvp -= C) {
                 if (FULL || i < cnt) {
                     const float ys = in.ys[i][lane], iden = in.iden[i][lane], ec = in.ec[i][lane], nm = in.neg_m[i][lane];
-                    const float direct = gg[i] * iden * ec;
-                    const float later = __expf(kk[i] + go);
-                    *gkp = from_float<T>(direct * (vv[i] - ys) + later * (gp * vv[i] + gq));
+                    const float ki = to_float(kk[i]), vi = to_float(vv[i]), gi = to_float(gg[i]);
+                    const float direct = gi * iden * ec;
+                    const float later = __expf(ki + go);
+                    *gkp = from_float<T>(direct * (vi - ys) + later * (gp * vi + gq));
                     *gvp = from_float<T>(direct + later * gp);
                     const float wg = w + go;
                     const ExpPair e = exp_pair(wg, nm);      // gy_t / den_t carries the exponent -m_t
-                    const float add = gg[i] * iden * e.second;
+                    const float add = gi * iden * e.second;
                     gp = fmaf(e.first, gp, add);
                     gq = fmaf(e.first, gq, -add * ys);
                     go = e.first_is_max ? wg : nm;
                 }
             }
         };
-        auto step = [&](int j, float (&kk)[CK], float (&vv)[CK], float (&gg)[CK], const V4Replay &in) {
+        auto step = [&](int j, T (&kk)[CK], T (&vv)[CK], T (&gg)[CK], const V4Replay &in) {
             const int blk = nblk - j;
             if (j >= 1) {
                 if ((blk + 1) * CK <= Tlen) walk(std::true_type{}, blk, kk, vv, gg, in);
