@@ -1,3 +1,5 @@
+import os
+
 import torch
 
 
@@ -9,6 +11,8 @@ def assert_close(got, ref, rtol, name=""):
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
     err = (got - ref).abs()
     bound = rtol * ref.abs() + rtol * ref.pow(2).mean().sqrt()
+    if os.environ.get("WKV_SHOW_MARGIN"):       # worst error as a fraction of what the tolerance allows
+        print(f"margin {name}: {(err / bound).max().item():.3f}", flush=True)
     bad = err > bound
     if bad.any():
         i = torch.argmax(err - bound)
