@@ -499,3 +499,52 @@ def test_plan_may_change_between_forward_and_backward(nseg_fwd, nseg_bwd):
     got = dict(y=y, state=s, gr=leaves["r"].grad, gk=leaves["k"].grad, gv=leaves["v"].grad, gw=leaves["w"].grad,
                gu=leaves["u"].grad, gstate=leaves["state"].grad)
     compare(got, run_oracle56(6, wl), 2e-2, f"plan {nseg_fwd}->{nseg_bwd}")
+
+
+def _sweep_cases():
+    """Seeded random shapes and decay regimes for the blocked path: ragged lengths, one to seven heads, forced and
+    automatic time splits with forced piece lengths, fast / slow / mixed / floored decays, with and without a state
+    gradient arriving."""
+    import random
+    rnd = random.Random(20240611)
+    cases = []
+    for i in range(24):
+        version = 5 if i % 3 == 0 else 6
+        B, H = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 3, 5, 7])
+        T = rnd.choice([rnd.randint(2, 63), rnd.randint(64, 400), rnd.randint(401, 1500), 64 * rnd.randint(1, 20)])
+        nseg = rnd.choice([0, 1, 2, 3, 5])
+        pps = rnd.choice([0, 0, 1, 3])
+        regime = rnd.choice(["fast", "slow", "mixed", "floor"])
+        cases.append((i, version, B, H, T, nseg, pps, regime, rnd.random() < 0.75))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: f"{c[0]}-v{c[1]}-B{c[2]}H{c[3]}T{c[4]}-n{c[5]}p{c[6]}-{c[7]}")
+def test_chunked_random_sweep(case):
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    i, version, B, H, T, nseg, pps, regime, with_gstate = case
+    wl = configs.make(1 if version == 5 else 3, B=B, T=T, C=64 * H, H=H, dtype=torch.bfloat16, seed=5000 + i)
+    w = wl.tensors["w"]
+    g = torch.Generator().manual_seed(7000 + i)
+    if regime == "slow":
+        w -= 4.0 if version == 6 else 0.0            # (WKV5 draws its decay from U(-6, 0): slow channels are in it already)
+    elif regime == "mixed":
+        mask = torch.rand(w.shape[-1] if version == 6 else w.shape, generator=g) < 0.5
+        w[..., mask] -= 4.5 if version == 6 else 0.0
+        if version == 5:
+            w[mask] -= 2.0
+    elif regime == "floor":
+        hit = torch.rand(w.shape, generator=g) < 0.05
+        w[hit] = 2.5                                  # exp(-exp(2.5)) = 5e-6: held at the floor of 0.005
+    print(f"case sweep {case}", flush=True)
+    assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg) == 0 and L.wkv_tune(_lib.TUNE_PIECE_STEPS, pps) == 0
+    try:
+        got = run_gpu56(version, wl, with_gstate=with_gstate, algo="chunked")
+    finally:
+        assert L.wkv_tune(_lib.TUNE_SEGMENTS, 0) == 0 and L.wkv_tune(_lib.TUNE_PIECE_STEPS, 0) == 0
+    ref = run_oracle56(version, wl, with_gstate=with_gstate)
+    compare(got, ref, 2e-2, f"sweep {case}")              # bf16 I/O: rtol 2e-2, floor 2e-2 rms
+    if regime == "floor":
+        hit_gw = got["gw"].float().cpu()[hit]
+        assert (hit_gw == 0).all(), "no gradient where the floor holds"
