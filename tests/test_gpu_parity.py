@@ -427,7 +427,8 @@ def test_chunked_time_segments_slow_decay(kind, nseg, pps):
 
 
 @pytest.mark.parametrize("nseg,T", [(1, 200), (3, 1000)])
-def test_chunked_v6_takes_bf16_decay(nseg, T):
+@pytest.mark.parametrize("shift", [0.0, -5.0])
+def test_chunked_v6_takes_bf16_decay(nseg, T, shift):
     """The raw decay handed over in bf16 (what a mixed-precision TimeMix produces and the reference widens with
     w.float(), RWKV-v6/src/module/TimeMix.py:50) is read as it is by the blocked kernels, and its gradient comes
     back in bf16 (as the reference allocates it, :90): same results as the oracle on the widened tensor."""
@@ -435,8 +436,8 @@ def test_chunked_v6_takes_bf16_decay(nseg, T):
     from rwkv_wkv_hip import _lib, configs
     L = _lib.lib()
     wl = configs.make(3, B=2, T=T, C=128, H=2, dtype=torch.bfloat16)
-    wl.tensors["w"] = wl.tensors["w"].to(torch.bfloat16)
-    print(f"case bf16 decay nseg={nseg} T={T}", flush=True)
+    wl.tensors["w"] = (wl.tensors["w"] + shift).to(torch.bfloat16)          # (shift -5: no piece of the split's passes stops early)
+    print(f"case bf16 decay nseg={nseg} T={T} shift={shift}", flush=True)
     assert L.wkv_tune(_lib.TUNE_SEGMENTS, nseg) == 0
     try:
         got = run_gpu56(6, wl, algo="chunked")

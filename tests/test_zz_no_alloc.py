@@ -110,3 +110,38 @@ def test_state_in_place_where_no_sequence_is_cut():
     assert fwd(_lib.ALGO_CHUNKED, one, one, 4)[0] == -8                 # cut in time: two buffers needed
     big = torch.zeros(2 * g["state"].numel(), device="cuda")
     assert fwd(_lib.ALGO_RECURRENT, big[:g["state"].numel()], big[64:64 + g["state"].numel()], 1)[0] == -8      # partial overlap
+
+
+def test_noalloc_forward_under_graph_capture():
+    """What the entry point is for: recorded into a HIP graph (after wkv_init, nothing is left to set up inside the
+    capture) and replayed, with plain launches in between; every replay gives the bits of the plain call."""
+    from rwkv_wkv_hip import _lib, configs
+    L = _lib.lib()
+    assert L.wkv_init() == 0
+    B, T, H = 1, 1024, 3
+    C = H * 64
+    wl = configs.make(3, seed=15, B=B, T=T, C=C, H=H, dtype=torch.bfloat16)
+    g = {n: x.cuda().contiguous() for n, x in wl.tensors.items()}
+    p = lambda t: t.data_ptr()
+    y, s = torch.empty_like(g["r"]), torch.empty_like(g["state"])
+
+    def call(stream):
+        st = L.wkv6_forward_noalloc(stream, B, T, C, H, _lib.WKV_BF16, _lib.FLOOR_DECAY, p(g["r"]), p(g["k"]), p(g["v"]),
+                                    p(g["w"]), p(g["u"]), p(g["state"]), p(y), p(s))
+        assert st == 0, L.wkv_strerror(st)
+    call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want = (y.clone(), s.clone())
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        y.fill_(3.0); s.fill_(3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[0]) and torch.equal(s, want[1]), f"replay {rep} differs"
+        call(torch.cuda.current_stream().cuda_stream)          # the program's own work between the replays
+        torch.cuda.synchronize()
