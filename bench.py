@@ -464,6 +464,21 @@ def bench_edges(a):
         timed(f"{tag} shift_mix v6 backward (5 mixes + data-dependent part)", mk(lambda s: L.wkv_shift_mix_backward(
             stream, B, T, C, 1, 5, 0, p(s["x"]), p(s["shift"]), p(coef), p(s["dyn"]), arr(s["o"]), p(s["gx"]), p(s["gshift"]), p(gcoef),
             p(s["gdyn"]), p(ws), ws.numel())), 34 * E)
+        # the same five mixes with the second LoRA product inside the pass: x and the activations in, five mixes out
+        # (backward: x, five gradients in; gx and the five product gradients out); the 32-wide activations and
+        # factors are 160 / 4096 of a tensor each and are counted
+        act = [torch.tanh(torch.randn(B * T, 5, 32, device="cuda")).to(bf) for _ in range(rot)]
+        w2t = (torch.randn(5, C, 32, device="cuda") * 0.1).to(bf)
+        ws2 = torch.empty(L.wkv_lora_mix_backward_workspace(B, T, C), dtype=torch.uint8, device="cuda")
+        small = 2 * (B * T * 160 + 160 * C)
+        timed(f"{tag} lora_mix v6 forward (5 mixes, LoRA product inside)", [
+            (lambda s=s, a_=a_: L.wkv_lora_mix_forward(stream, B, T, C, p(s["x"]), p(s["shift"]), p(coef), p(a_), p(w2t), arr(s["o"])))
+            for s, a_ in zip(sets, act)], 12 * E + small)
+        timed(f"{tag} lora_mix v6 backward (5 mixes, LoRA product inside)", [
+            (lambda s=s, a_=a_: L.wkv_lora_mix_backward(stream, B, T, C, p(s["x"]), p(s["shift"]), p(coef), p(a_), p(w2t), arr(s["o"]),
+                                                        p(s["gx"]), p(s["gshift"]), p(gcoef), p(s["gdyn"]), p(ws2), ws2.numel()))
+            for s, a_ in zip(sets, act)], 24 * E + small)
+        del act
         timed(f"{tag} ln_x * gate forward", mk(lambda s: L.wkv_ln_gate_forward(
             stream, B * T, C, 1, 1.0, 64e-5, p(s["x"]), p(s["o"][0]), p(wb[0]), p(wb[1]), p(s["gx"]))), 6 * E)
         timed(f"{tag} ln_x * gate backward", mk(lambda s: L.wkv_ln_gate_backward(
@@ -569,6 +584,9 @@ def bench_block(a):
     if a.block_way in ("both", "kernels"):
         timed("timemix_kernels_ms", lambda: K.timemix6_forward(tm, x, (shift, state))[0])
         timed("channelmix_kernels_ms", lambda: K.channelmix6_forward(cm, x, shift)[0])
+        K.use_lora_mix(False)       # the same with the second LoRA product and its five results through memory
+        timed("timemix_kernels_lora_through_memory_ms", lambda: K.timemix6_forward(tm, x, (shift, state))[0])
+        K.use_lora_mix(True)
     if a.block_way in ("both", "torch"):
         timed("timemix_torch_elementwise_ms", lambda: timemix_torch(tm, x, (shift, state))[0])
         timed("channelmix_torch_elementwise_ms", lambda: channelmix_torch(cm, x, shift)[0])

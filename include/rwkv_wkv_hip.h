@@ -236,6 +236,25 @@ int wkv_shift_mix_backward(void *stream, int B, int T, int C, int dtype, int n, 
                            const void *shift, const float *coef, const void *dyn, const void *const *gout, void *gx,
                            void *gshift, float *gcoef, void *gdyn, void *workspace, size_t workspace_bytes);
 
+/* The data-dependent mix of the v6 TimeMix with its second LoRA product inside the pass
+ * (RWKV-v6/src/module/TimeMix.py:264-276; replaces `torch.bmm(xxx, self.time_maa_w2)` of :265 and the five mixes of
+ * :269-273, whose operands mw, mk, mv, mr, mg are then never written to memory):
+ *   out[j][b,t,:] = x[b,t,:] + (x[b,t-1,:] - x[b,t,:]) * (coef[j] + act[b*T+t, j, :] @ w2[j]),   j < 5 = w, k, v, r, g
+ * bf16 only.  x (B,T,C); shift (B,C); coef (5,C) fp32 = time_maa_w, _k, _v, _r, _g; act (B*T, 5, 32) =
+ * tanh(xxx @ time_maa_w1) as the reference views it before its transpose (:264); w2t (5, C, 32) = time_maa_w2 with its
+ * last two dimensions exchanged; out: HOST array of 5 device pointers, each (B,T,C).  C a multiple of 8. */
+int wkv_lora_mix_forward(void *stream, int B, int T, int C, const void *x, const void *shift, const float *coef,
+                         const void *act, const void *w2t, void *const *out);
+
+/* Its backward: gout = HOST array of the 5 output gradients; gx (B,T,C), gshift (B,C) bf16; gcoef (5,C) fp32, summed
+ * over batch and time in a fixed order; gdyn (5,B,T,C) bf16 = the gradients of the five products act @ w2[j] (what
+ * autograd hands to the backward of the reference's bmm: the gradients of act and of w2 are two matrix products with
+ * it, left to the caller's GEMM library).  workspace: wkv_lora_mix_backward_workspace bytes. */
+size_t wkv_lora_mix_backward_workspace(int B, int T, int C);
+int wkv_lora_mix_backward(void *stream, int B, int T, int C, const void *x, const void *shift, const float *coef,
+                          const void *act, const void *w2t, const void *const *gout, void *gx, void *gshift,
+                          float *gcoef, void *gdyn, void *workspace, size_t workspace_bytes);
+
 /* ln_x and the gate on the operator's output (RWKV-v5/src/module/TimeMix.py:301,317-320: scale = 1/8, eps = 1e-5;
  * RWKV-v6/src/module/TimeMix.py:180,278,296-298: scale = 1, eps = 64e-5):
  *   out = (GroupNorm(y * scale; one group per 64-channel head, eps) * weight + bias) * silu(gate)

@@ -8,6 +8,7 @@ is the reference's backward:
 ``modified_lerp``    RWKV-v5/src/module/OptimizedOps.py:14-15
 ``mix_v5``           RWKV-v5/src/module/TimeMix.py:295-298, ChannelMix.py:46-47
 ``mix_v6``           RWKV-v6/src/module/TimeMix.py:262-276, ChannelMix.py:33-35
+``lora_mix_v6``      RWKV-v6/src/module/TimeMix.py:264-273 (the second LoRA product and the five mixes it feeds)
 ``ln_x_gate``        RWKV-v5/src/module/TimeMix.py:301,317-320 (divisor 8, eps 1e-5);
                      RWKV-v6/src/module/TimeMix.py:180,278,296-298 (divisor 1, eps 64e-5)
 ``relu_square``, ``sigmoid_mul``   RWKV-v5/src/module/ChannelMix.py:48-49
@@ -16,7 +17,8 @@ is the reference's backward:
 
 Pinned by (tests/test_oracle_blocks.py): the mixes at coefficient 0 and 1 (identity / pure shift), token_shift against
 an index loop, ln_x_gate against a written-out mean/variance normalisation and against torch's layer_norm per head,
-L2Wrap against a per-row Python loop, the two activations against their textbook formulas in numpy.
+L2Wrap against a per-row Python loop, the two activations against their textbook formulas in numpy, lora_mix_v6
+against a per-token, per-mix loop of matrix-vector products (and against mix_v6 at w2 = 0).
 """
 from __future__ import annotations
 
@@ -45,6 +47,15 @@ def mix_v6(x, shift_state, maas, dyn=None):
     if dyn is None:
         return tuple(x + dxprev * m for m in maas)
     return tuple(x + dxprev * (m + d) for m, d in zip(maas, dyn.unbind(0)))
+
+
+def lora_mix_v6(x, shift_state, maas, act, w2):
+    """the reference's five data-dependent mixes from act = tanh(xxx @ time_maa_w1) as (B*T, 5, D) and
+    w2 = time_maa_w2 (5, D, C): the batched product of TimeMix.py:264-265 (transpose, bmm, view) and the mixes of
+    :269-273; maas = (time_maa_w, _k, _v, _r, _g); returns (xw, xk, xv, xr, xg)"""
+    B, T, C = x.shape
+    dyn = torch.bmm(act.transpose(0, 1), w2).view(5, B, T, -1)
+    return mix_v6(x, shift_state, maas, dyn)
 
 
 def ln_x_gate(y, gate, weight, bias, n_head, eps, divisor=1.0):

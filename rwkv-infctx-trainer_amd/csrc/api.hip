@@ -9,6 +9,7 @@
 #include "wkv4.hip"
 #include "cumsum_decay.hip"
 #include "block_edges.hip"
+#include "lora_mix.hip"
 
 using namespace wkv;
 
@@ -357,6 +358,49 @@ int wkv_shift_mix_backward(void *stream, int B, int T, int C, int dtype, int n, 
                                                  gcoef, gdyn, (float *)workspace)
     hipError_t e = WKV_BY_DTYPE(dtype, CALL);
 #undef CALL
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+static int lora_mix_dims(int B, int T, int C) {
+    if (B <= 0 || T <= 0 || C <= 0 || C % 8 != 0 || B > 65535) return WKV_ERR_DIMS;
+    if (edges::lora_mix_tiles(T) > 65535) return WKV_ERR_DIMS;          // rows of workgroups in one launch
+    return WKV_OK;
+}
+
+size_t wkv_lora_mix_backward_workspace(int B, int T, int C) {
+    if (lora_mix_dims(B, T, C) != WKV_OK) return 0;
+    return edges::lora_mix_backward_workspace(B, T, C);
+}
+
+int wkv_lora_mix_forward(void *stream, int B, int T, int C, const void *x, const void *shift, const float *coef,
+                         const void *act, const void *w2t, void *const *out) {
+    if (int e = lora_mix_dims(B, T, C)) return e;
+    if (!x || !shift || !coef || !act || !w2t || !out) return WKV_ERR_NULL;
+    for (int j = 0; j < edges::LM_N; j++) {
+        if (!out[j]) return WKV_ERR_NULL;
+        if (!aligned16(out[j])) return WKV_ERR_ALIGN;
+    }
+    for (const void *p : {x, shift, (const void *)coef, act, w2t})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    hipError_t e = edges::lora_mix_forward_launch((hipStream_t)stream, B, T, C, x, shift, coef, act, w2t, out);
+    return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
+}
+
+int wkv_lora_mix_backward(void *stream, int B, int T, int C, const void *x, const void *shift, const float *coef,
+                          const void *act, const void *w2t, const void *const *gout, void *gx, void *gshift, float *gcoef,
+                          void *gdyn, void *workspace, size_t workspace_bytes) {
+    if (int e = lora_mix_dims(B, T, C)) return e;
+    if (!x || !shift || !coef || !act || !w2t || !gout || !gx || !gshift || !gcoef || !gdyn || !workspace) return WKV_ERR_NULL;
+    for (int j = 0; j < edges::LM_N; j++) {
+        if (!gout[j]) return WKV_ERR_NULL;
+        if (!aligned16(gout[j])) return WKV_ERR_ALIGN;
+    }
+    for (const void *p : {x, shift, (const void *)coef, act, w2t, (const void *)gx, (const void *)gshift, (const void *)gcoef,
+                          (const void *)gdyn, (const void *)workspace})
+        if (!aligned16(p)) return WKV_ERR_ALIGN;
+    if (workspace_bytes < edges::lora_mix_backward_workspace(B, T, C)) return WKV_ERR_WORKSPACE;
+    hipError_t e = edges::lora_mix_backward_launch((hipStream_t)stream, B, T, C, x, shift, coef, act, w2t, gout, gx, gshift, gcoef,
+                                                   gdyn, (float *)workspace);
     return e == hipSuccess ? WKV_OK : WKV_ERR_LAUNCH;
 }
 

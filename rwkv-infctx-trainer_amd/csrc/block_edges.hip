@@ -32,6 +32,26 @@ template <class T> __device__ __forceinline__ void store8(T *p, const float (&o)
     store4(p, a); store4(p + 4, b);
 }
 
+// The same for a result that this pass does not read again: stored with the non-temporal hint, so that a tensor being
+// written does not push the tensors being read out of the last-level cache (5 to 25 % on these passes taken alone,
+// most at sizes near the cache's 256 MB).  The two channel-mix activations keep the plain store: their results are the
+// very next matrix product's operand, and a layer measured as a whole is 1 % slower when they bypass the cache.
+__device__ __forceinline__ void stream8(float *p, const float (&o)[8]) {
+    typedef float f4_ __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(f4_{o[0], o[1], o[2], o[3]}, reinterpret_cast<f4_ *>(p));
+    __builtin_nontemporal_store(f4_{o[4], o[5], o[6], o[7]}, reinterpret_cast<f4_ *>(p + 4));
+}
+__device__ __forceinline__ void stream8(bf16 *p, const float (&o)[8]) {
+    typedef unsigned int u4_ __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(u4_{bf16_pack2(o[0], o[1]), bf16_pack2(o[2], o[3]), bf16_pack2(o[4], o[5]), bf16_pack2(o[6], o[7])},
+                                reinterpret_cast<u4_ *>(p));
+}
+__device__ __forceinline__ void stream8(f16 *p, const float (&o)[8]) {
+    typedef _Float16 h8_ __attribute__((ext_vector_type(8)));
+    const h8_ x = {(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3], (_Float16)o[4], (_Float16)o[5], (_Float16)o[6], (_Float16)o[7]};
+    __builtin_nontemporal_store(x, reinterpret_cast<h8_ *>(p));
+}
+
 template <int N> struct Ptrs { void *p[N]; };
 template <int N> struct ConstPtrs { const void *p[N]; };
 
@@ -73,7 +93,7 @@ __global__ __launch_bounds__(256) void shift_mix_forward(int Tlen, int C, int le
 #pragma unroll
             for (int e = 0; e < 8; e++)
                 o[e] = fmaf(row[i][e] - row[i + 1][e], DYN ? cd[j][e] + d[e] : cd[j][e], row[i + 1][e]);
-            store8((T *)out.p[j] + off, o);
+            stream8((T *)out.p[j] + off, o);
         }
     }
 }
@@ -149,9 +169,9 @@ __global__ __launch_bounds__(256) void shift_mix_backward(int Tlen, int C, int l
                     d[e] = g[e] * dx[e];
                     acc[j][e] += d[e];
                 }
-                if (DYN) store8(gdyn + (size_t)j * plane + off, d);
+                if (DYN) stream8(gdyn + (size_t)j * plane + off, d);
             }
-            store8(gx + off, own);
+            stream8(gx + off, own);
 #pragma unroll
             for (int e = 0; e < 8; e++) carry[e] = next[e];
         }
@@ -255,7 +275,7 @@ __global__ __launch_bounds__(256) void ln_gate_forward(int rows, int C, float sc
                 const float n = fmaf(v[i][e] * rstd, w[e], bs[e]);
                 o[e] = gate ? n * g[i][e] * sigmoid_f(g[i][e]) : n;
             }
-            store8(out + (size_t)r * C + c, o);
+            stream8(out + (size_t)r * C + c, o);
         }
     }
 }
@@ -324,8 +344,8 @@ __global__ __launch_bounds__(256) void ln_gate_backward(int rows, int C, float s
             float o[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) o[e] = scale * rstd * (go[e] - m1 - v[e] * m2);
-            store8(gy + off, o);
-            if (gate) store8(ggate + off, gg);
+            stream8(gy + off, o);
+            if (gate) stream8(ggate + off, gg);
         }
     }
 #pragma unroll
@@ -429,7 +449,7 @@ __global__ __launch_bounds__(256) void l2wrap_backward(int V, float factor, cons
             float o[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) o[e] = (i + e == bi) ? val : 0.f;
-            store8(gy + base + i, o);
+            stream8(gy + base + i, o);
         }
     } else {
         for (int i = threadIdx.x; i < V; i += 256) gy[base + i] = from_float<T>(i == bi ? val : 0.f);

@@ -24,6 +24,11 @@
 
 namespace wkv {
 
+// one element of a result, stored with the non-temporal hint (results are not read again by these kernels)
+__device__ __forceinline__ void stream1(float *p, float v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void stream1(bf16 *p, bf16 v) { __builtin_nontemporal_store(v.bits, &p->bits); }
+__device__ __forceinline__ void stream1(f16 *p, f16 v) { __builtin_nontemporal_store(v.h, &p->h); }
+
 constexpr int CK = 16;                 // tokens per checkpoint block
 constexpr float NEG_HUGE = -1e38f;
 
@@ -115,7 +120,7 @@ __global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const 
                     if (decltype(full)::value || i < cnt) {
                         float iden, ec, hw, nm;
                         const float yy = v4_step(s, w, u, to_float(bk[d][i]), to_float(bv[d][i]), iden, ec, hw, nm);
-                        if (decltype(with_y)::value) { *yp = from_float<T>(yy); yp += C; }
+                        if (decltype(with_y)::value) { stream1(yp, from_float<T>(yy)); yp += C; }
                     }
                 }
             };
@@ -247,8 +252,8 @@ __global__ __launch_bounds__(128) void v4_backward(int BC, int Tlen, int C, cons
                     const float ki = to_float(kk[i]), vi = to_float(vv[i]), gi = to_float(gg[i]);
                     const float direct = gi * iden * ec;
                     const float later = __expf(ki + go);
-                    *gkp = from_float<T>(direct * (vi - ys) + later * (gp * vi + gq));
-                    *gvp = from_float<T>(direct + later * gp);
+                    stream1(gkp, from_float<T>(direct * (vi - ys) + later * (gp * vi + gq)));
+                    stream1(gvp, from_float<T>(direct + later * gp));
                     const float wg = w + go;
                     const ExpPair e = exp_pair(wg, nm);      // gy_t / den_t carries the exponent -m_t
                     const float add = gi * iden * e.second;

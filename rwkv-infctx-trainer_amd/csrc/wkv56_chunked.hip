@@ -52,10 +52,12 @@ namespace chunked {
 #define PT_DECL long long pt_[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long pt_last_ = clock64();
 #define PT_MARK(i) { const long long now_ = clock64(); pt_[i] += now_ - pt_last_; pt_last_ = now_; }
 #define PT_PRINT(name) if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) printf("%s[%d]: p0 %lld p1 %lld p2 %lld p3 %lld p4 %lld p5 %lld p6 %lld p7 %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5], pt_[6], pt_[7]);
+#define PT_PRINT_WAVES(name) if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) printf("%s[%d]: p0 %lld p1 %lld p2 %lld p3 %lld p4 %lld\n", name, (int)threadIdx.x, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4]);
 #else
 #define PT_DECL
 #define PT_MARK(i)
 #define PT_PRINT(name)
+#define PT_PRINT_WAVES(name)
 #endif
 
 // (lds_barrier(): the workgroup barrier of these kernels, whose wavefronts talk to each other through LDS alone)
@@ -195,7 +197,8 @@ constexpr int PART = HEAD * HEAD + HEAD;
 //   chains    wavefronts 0-7 own the state for good: wavefront (w, half) holds keys
 //             32*half..32*half+31 x values 16w..16w+15 in registers, walks it over the four
 //             blocks and leaves its share of  rh S  per block in LDS;
-//             wavefronts 8-11 build the masked intra-block matrix of one block each.
+//             wavefronts 8-15 build the masked intra-block matrix of one block each, one half of the
+//             keys a wavefront (the two parts are added by the MFMAs of the finish).
 //   finish    wavefront (q, w): y of block q, value columns 16w..16w+15 = the two shares
 //             + (intra-block matrix) v, converted and stored.
 constexpr int NT_F16 = 1024;
@@ -209,7 +212,7 @@ struct Fwd16Tiles {
     float dec[4][HEAD];       // e^{b} per block and key
     float ent[4][HEAD];       // e^{-b}
     float rho[SB];            // r . (u o k) per token
-    uint4 amat[4][64];        // masked intra-block matrix of each block as A-operand fragments (head, remainder)
+    uint4 amat[2][4][64];     // masked intra-block matrix of each block, one part per half of the keys, as A-operand fragments (head, remainder)
     float4 yi[2][4][4][64];   // rh S per key half, block, value quarter: accumulator layout, one float4 per lane
     float wtot[16][HEAD];     // per wavefront (four tokens) and channel: sum of log w, for the block-wide running sum
 };
@@ -371,6 +374,7 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
     if (tid < HEAD) sm.fac[0][tid] = 1.f;
     if (tid == 0) sm.stop = 0;
     bool stopped = false;
+    PT_DECL
     for (int it = 0; it < nsteps; it++) {
         const int par = it & 1;
         {
@@ -417,16 +421,16 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
                 *reinterpret_cast<float4 *>(&sm.dec[wv][c4]) = make_float4(exp2_fast(tot[0]), exp2_fast(tot[1]), exp2_fast(tot[2]), exp2_fast(tot[3]));
             }
         }
+        PT_MARK(0)
         lds_barrier();
+        PT_MARK(1)
         if (it + 1 < nsteps) fetch(step_at(it + 1));          // next step's loads fly during the MFMA phase
         if (wv == 0) {      // lane = key: the decay up to the next step, and whether anything later can still matter
             R += (sm.tot[0][lane] + sm.tot[1][lane]) + (sm.tot[2][lane] + sm.tot[3][lane]);
             sm.fac[par ^ 1][lane] = exp2_fast(R);
-            float mx = R;
-#pragma unroll
-            for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-            if (lane == 0 && mx < PASS_CUT_LOG2) sm.stop = 1;
+            if (__builtin_amdgcn_ballot_w64(R >= PASS_CUT_LOG2) == 0 && lane == 0) sm.stop = 1;
         }
+        PT_MARK(2)
         // the step's own contribution, its four blocks chained from zero (first to last going forward, last to first going back)
         f4 Tt[4];
 #pragma unroll
@@ -451,9 +455,12 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
             X[kk][0] = fmaf(f.x, Tt[kk][0], X[kk][0]); X[kk][1] = fmaf(f.y, Tt[kk][1], X[kk][1]);
             X[kk][2] = fmaf(f.z, Tt[kk][2], X[kk][2]); X[kk][3] = fmaf(f.w, Tt[kk][3], X[kk][3]);
         }
+        PT_MARK(3)
         lds_barrier();
+        PT_MARK(4)
         if (sm.stop) { stopped = true; break; }
     }
+    PT_PRINT_WAVES(BACKWARD ? "gradient summary" : "state summary")
     float *pp = part + ((size_t)bh * nseg * m + piece) * PART;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
@@ -523,7 +530,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     const int bh = bh0 + blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
     const int q = w16 >> 2, wv = w16 & 3;          // block and quarter for preparing and finishing
-    const bool chain = w16 < 8, builder = w16 >= 8 && w16 < 12;
+    const bool chain = w16 < 8;                    // the other eight build the intra-block matrices: block wv, key half (w16 >> 2) & 1
     const int hk = w16 >> 2;                       // chain wavefronts: key half
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int nsb = (Tlen + SB - 1) / SB;
@@ -695,14 +702,14 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
                 y0 += y1 + y2;
                 sm.yi[hk][blk][wv][lane] = make_float4(y0[0], y0[1], y0[2], y0[3]);
             }
-        } else if (builder) {
-            // ---------------- the masked intra-block matrix of block wv, once for everybody:
+        } else {
+            // ---------------- the masked intra-block matrix of block wv, once for everybody, as the sum of two
+            // matrices (one per half of the keys, each by its own wavefront):
             // A^T[s][t] = sum_i (k e^{b-incl})[s][i] (r e^{excl-b})[t][i]; lane gets s = 4g+e, t = n
-            const int row = 16 * wv + n;
+            const int row = 16 * wv + n, kh2 = (w16 >> 2) & 1;
             f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
-#pragma unroll
-            for (int kk = 0; kk < 4; kk += 2) {
-                const int ca = 16 * kk + 4 * g, cb = ca + 16;
+            {
+                const int ca = 32 * kh2 + 4 * g, cb = ca + 16;
                 const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb);
                 s4 r0, r1, r0l, r1l;
                 scale_split(frag(sm.rh, row, ca), frag(sm.rhl, row, ca), *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), n == 0, r0, r0l);
@@ -712,7 +719,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
                 a2 = mma2(k0, k1, r0l, r1l, a2);
             }
             f4 at = a0 + (a1 + a2);
-            const float rho_t = sm.rho[row];
+            const float rho_t = kh2 ? 0.f : sm.rho[row];       // the diagonal goes with the first half
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int s_ = 4 * g + e;
@@ -721,7 +728,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             uint32_t h0, l0, h1, l1;                        // A[t = n][s = 4g..4g+3] as head + remainder
             split2(at[0], at[1], h0, l0);
             split2(at[2], at[3], h1, l1);
-            sm.amat[wv][lane] = make_uint4(h0, h1, l0, l1);
+            sm.amat[kh2][wv][lane] = make_uint4(h0, h1, l0, l1);
         }
         PT_MARK(2)
         lds_barrier();
@@ -730,10 +737,11 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
         // ---------------- y of block q, value columns 16wv..16wv+15
         if (y) {
             const float4 ya = sm.yi[0][q][wv][lane], yb = sm.yi[1][q][wv][lane];
-            const uint4 am = sm.amat[q][lane];
+            const uint4 am = sm.amat[0][q][lane], am2 = sm.amat[1][q][lane];
             const s4 v_op = frag_tr(sm.v, tro + (16 * q) * LD + 16 * wv);
             f4 yt = {ya.x + yb.x, ya.y + yb.y, ya.z + yb.z, ya.w + yb.w};
             yt = mma2(as_s4(am.x, am.y), as_s4(am.z, am.w), v_op, v_op, yt);
+            yt = mma2(as_s4(am2.x, am2.y), as_s4(am2.z, am2.w), v_op, v_op, yt);
             // into the rh tile (nobody reads it any more in this step), [token][value]; it leaves as full rows
 #pragma unroll
             for (int e = 0; e < 4; e++) sm.rh[(16 * q + 4 * g + e) * LD + 16 * wv + n] = bf16_bits(yt[e]);

@@ -49,6 +49,9 @@ SIGNATURES = {
     "wkv_shift_mix_forward": (_I, [_P, _I, _I, _I, _I, _I, _I] + [_P] * 5),
     "wkv_shift_mix_backward_workspace": (c_size_t, [_I] * 4),
     "wkv_shift_mix_backward": (_I, [_P, _I, _I, _I, _I, _I, _I] + [_P] * 9 + [_P, c_size_t]),
+    "wkv_lora_mix_forward": (_I, [_P, _I, _I, _I] + [_P] * 6),
+    "wkv_lora_mix_backward_workspace": (c_size_t, [_I] * 3),
+    "wkv_lora_mix_backward": (_I, [_P, _I, _I, _I] + [_P] * 10 + [_P, c_size_t]),
     "wkv_ln_gate_forward": (_I, [_P, _I, _I, _I, c_float, c_float] + [_P] * 5),
     "wkv_ln_gate_backward_workspace": (c_size_t, [_I] * 2),
     "wkv_ln_gate_backward": (_I, [_P, _I, _I, _I, c_float, c_float] + [_P] * 8 + [_P, c_size_t]),

@@ -4,6 +4,8 @@ and the block forwards that use them.
   token_shift_mix   token shift + mixing of the block input, any number of mixed copies from one read of x
                     (RWKV-v5/src/module/TimeMix.py:292-298, ChannelMix.py:44-47; RWKV-v6/src/module/TimeMix.py:262-276,
                     ChannelMix.py:31-35)
+  lora_shift_mix    the five data-dependent mixes of the v6 TimeMix with the second LoRA product inside the pass
+                    (RWKV-v6/src/module/TimeMix.py:264-276)
   ln_x_gate         GroupNorm per head times the SiLU gate (RWKV-v5 TimeMix.py:301,317-320; RWKV-v6 :278,296-298)
   relu_square, sigmoid_mul   channel-mix activations (RWKV-v5/src/module/ChannelMix.py:48-49)
   L2Wrap            RWKV-v5/src/model.py:123-148
@@ -25,6 +27,7 @@ from ._lib import check
 from .ops import _DT, _on_gpu, _ptr, _stream, _workspace, WKV_5, WKV_6
 
 MAX_MIX = 5
+LORA_MIXES, LORA_DIM = 5, 32      # the v6 TimeMix: five mixes, TIME_MIX_EXTRA_DIM = 32
 
 
 def _ptr_array(ts):
@@ -85,6 +88,71 @@ def token_shift_mix(x, shift_state, coefs, dyn=None, lerp=False):
     C = x.shape[-1]
     coef = torch.stack([c.reshape(C).float() for c in coefs], 0)
     return _ShiftMix.apply(bool(lerp), x, shift_state, coef, dyn)
+
+
+class _LoraMix(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, shift, coef, act, w2):
+        """coef (5, C) fp32; act (B*T, 5, 32); w2 (5, 32, C); returns 5 tensors (B, T, C)"""
+        _on_gpu(x, shift, coef, act, w2)
+        B, T, C = x.shape
+        assert x.dtype == torch.bfloat16 and act.dtype == x.dtype and w2.dtype == x.dtype
+        assert coef.shape == (LORA_MIXES, C) and coef.dtype == torch.float32
+        assert act.shape == (B * T, LORA_MIXES, LORA_DIM) and w2.shape == (LORA_MIXES, LORA_DIM, C)
+        x, act = x.contiguous(), act.contiguous()
+        shift = shift.to(x.dtype).contiguous()
+        w2t = w2.transpose(1, 2).contiguous()                    # (5, C, 32): a channel's 32 factors side by side
+        outs = [torch.empty_like(x) for _ in range(LORA_MIXES)]
+        check(_lib.lib().wkv_lora_mix_forward(_stream(), B, T, C, _ptr(x), _ptr(shift), _ptr(coef), _ptr(act), _ptr(w2t),
+                                              _ptr_array(outs)), "wkv_lora_mix_forward")
+        ctx.save_for_backward(x, shift, coef, act, w2t)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *gouts):
+        x, shift, coef, act, w2t = ctx.saved_tensors
+        B, T, C = x.shape
+        gouts = [torch.zeros_like(x) if g is None else g.to(x.dtype).contiguous() for g in gouts]
+        gx = torch.empty_like(x)
+        gshift = torch.empty_like(shift)
+        gcoef = torch.empty_like(coef)
+        gdyn = torch.empty((LORA_MIXES, B * T, C), dtype=x.dtype, device=x.device)
+        L = _lib.lib()
+        ws = _workspace(L.wkv_lora_mix_backward_workspace(B, T, C), x.device)
+        check(L.wkv_lora_mix_backward(_stream(), B, T, C, _ptr(x), _ptr(shift), _ptr(coef), _ptr(act), _ptr(w2t),
+                                      _ptr_array(gouts), _ptr(gx), _ptr(gshift), _ptr(gcoef), _ptr(gdyn), _ptr(ws), ws.numel()),
+              "wkv_lora_mix_backward")
+        # the two reductions of the product's backward: over the channels for act, over the tokens for w2
+        gact = torch.bmm(gdyn, w2t).transpose(0, 1)                               # (B*T, 5, 32)
+        gw2 = torch.bmm(act.permute(1, 2, 0), gdyn)                               # (5, 32, C)
+        return gx, gshift, gcoef, gact, gw2
+
+
+def lora_shift_mix(x, shift_state, coefs, act, w2):
+    """The five data-dependent mixes of the v6 TimeMix (RWKV-v6/src/module/TimeMix.py:264-276) from one read of x:
+    out_j = x + (xx - x) * (maa_j + act[:, j] @ w2[j]),  xx the sequence shifted by one token;
+    coefs = (time_maa_w, _k, _v, _r, _g); act (B*T, 5, 32) = tanh(xxx @ time_maa_w1) viewed as the reference views it;
+    w2 = time_maa_w2 (5, 32, C).  The products act[:, j] @ w2[j] (the reference's mw, mk, mv, mr, mg) stay inside the
+    kernel.  bf16, C a multiple of 8."""
+    C = x.shape[-1]
+    coef = torch.stack([c.reshape(C).float() for c in coefs], 0)
+    return _LoraMix.apply(x, shift_state, coef, act, w2)
+
+
+_lora_mix_on = True
+
+
+def use_lora_mix(on):
+    """timemix6_forward with (default) or without the fused pass, for comparisons; returns the previous setting"""
+    global _lora_mix_on
+    prev, _lora_mix_on = _lora_mix_on, bool(on)
+    return prev
+
+
+def lora_mix_available(x, act, w2):
+    """whether lora_shift_mix takes these operands (else: bmm + token_shift_mix with dyn)"""
+    return (_lora_mix_on and x.dtype == torch.bfloat16 and act.dtype == x.dtype and w2.dtype == x.dtype and x.shape[-1] % 8 == 0
+            and act.shape[-1] == LORA_DIM and act.shape[-2] == LORA_MIXES)
 
 
 class _LnGate(torch.autograd.Function):
@@ -223,10 +291,13 @@ def timemix6_forward(self, x, last_state):
     B, T, C = x.shape
     H = self.n_head
     (xxx,) = token_shift_mix(x, last_state[0], (self.time_maa_x,))
-    xxx = torch.tanh(xxx @ self.time_maa_w1).view(B * T, 5, -1).transpose(0, 1)
-    dyn = torch.bmm(xxx, self.time_maa_w2).view(5, B, T, C)                     # mw, mk, mv, mr, mg
-    xw, xk, xv, xr, xg = token_shift_mix(
-        x, last_state[0], (self.time_maa_w, self.time_maa_k, self.time_maa_v, self.time_maa_r, self.time_maa_g), dyn=dyn)
+    act = torch.tanh(xxx @ self.time_maa_w1).view(B * T, 5, -1)
+    maas = (self.time_maa_w, self.time_maa_k, self.time_maa_v, self.time_maa_r, self.time_maa_g)
+    if lora_mix_available(x, act, self.time_maa_w2):
+        xw, xk, xv, xr, xg = lora_shift_mix(x, last_state[0], maas, act, self.time_maa_w2)
+    else:       # other dtypes / LoRA sizes: the products through memory
+        dyn = torch.bmm(act.transpose(0, 1), self.time_maa_w2).view(5, B, T, C)                 # mw, mk, mv, mr, mg
+        xw, xk, xv, xr, xg = token_shift_mix(x, last_state[0], maas, dyn=dyn)
     r, k, v, gate = self.receptance(xr), self.key(xk), self.value(xv), self.gate(xg)
     # w = time_decay + tanh(xw @ w1) @ w2 (TimeMix.py:280-281): the broadcast addition rides on the second matmul as
     # its bias epilogue instead of being a pass of its own over (B,T,C)

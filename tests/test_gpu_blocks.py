@@ -62,6 +62,62 @@ def test_token_shift_mix(dtype, B, T, C, n, lerp, dyn):
         assert_close(got[4], ref[4], rt, "gdyn")
 
 
+@pytest.mark.parametrize("B,T,C", [(1, 1, 32), (2, 7, 96), (3, 130, 64), (2, 128, 2560), (1, 200, 320), (2, 129, 32),
+                                   (1, 257, 128), (2, 16, 4096)])
+def test_lora_shift_mix(B, T, C):
+    """The five data-dependent mixes with the second LoRA product inside the kernel (bf16) against the oracle in fp32
+    on the same rounded inputs: the five outputs and the gradients of x, the shift state, the five time_maa
+    parameters, the activations and time_maa_w2."""
+    from rwkv_wkv_hip import blocks as K
+    bf = torch.bfloat16
+    g = _g(B * 1000 + T + C)
+    x = torch.randn(B, T, C, generator=g).to(bf)
+    shift = torch.randn(B, C, generator=g).to(bf)
+    coefs = [torch.rand(1, 1, C, generator=g) for _ in range(5)]
+    act = torch.tanh(torch.randn(B * T, 5, 32, generator=g)).to(bf)
+    w2 = (torch.randn(5, 32, C, generator=g) * 0.1).to(bf)
+    gouts = [torch.randn(B, T, C, generator=g).to(bf) for _ in range(5)]
+
+    def run(fn, dev):
+        xs, ss, as_, ws = (_leaf(t.to(dev)) for t in (x, shift, act, w2))
+        cs = [_leaf(c.to(dev)) for c in coefs]
+        outs = fn(xs, ss, cs, as_, ws)
+        torch.autograd.backward(list(outs), [go.to(dev).to(outs[0].dtype) for go in gouts])
+        return outs, xs.grad, ss.grad, [c.grad for c in cs], as_.grad, ws.grad
+
+    ref = run(lambda xs, ss, cs, as_, ws: OB.lora_mix_v6(xs.float(), ss.float(), cs, as_.float(), ws.float()), "cpu")
+    assert K.lora_mix_available(x, act, w2)
+    got = run(lambda xs, ss, cs, as_, ws: K.lora_shift_mix(xs, ss, cs, as_, ws), "cuda")
+    torch.cuda.synchronize()
+    for j in range(5):
+        assert got[0][j].dtype == bf
+        assert_close(got[0][j], ref[0][j], 2e-2, f"out[{j}]")
+        assert_close(got[3][j], ref[3][j], 2e-2, f"gmaa[{j}]")
+    assert_close(got[1], ref[1], 2e-2, "gx")
+    assert_close(got[2], ref[2], 2e-2, "gshift")
+    assert_close(got[4], ref[4], 2e-2, "gact")
+    assert_close(got[5], ref[5], 2e-2, "gw2")
+
+
+def test_lora_shift_mix_matches_the_unfused_passes():
+    """the fused pass against bmm + token_shift_mix on the same device: the same mathematics with dyn rounded to bf16
+    on its way through memory in the one and kept in fp32 in the other"""
+    from rwkv_wkv_hip import blocks as K
+    bf = torch.bfloat16
+    B, T, C = 2, 200, 256
+    g = _g(5)
+    x, shift = torch.randn(B, T, C, generator=g).to(bf).cuda(), torch.randn(B, C, generator=g).to(bf).cuda()
+    coefs = [torch.rand(1, 1, C, generator=g).cuda() for _ in range(5)]
+    act = torch.tanh(torch.randn(B * T, 5, 32, generator=g)).to(bf).cuda()
+    w2 = (torch.randn(5, 32, C, generator=g) * 0.1).to(bf).cuda()
+    with torch.no_grad():
+        fused = K.lora_shift_mix(x, shift, coefs, act, w2)
+        dyn = torch.bmm(act.transpose(0, 1), w2).view(5, B, T, C)
+        plain = K.token_shift_mix(x, shift, coefs, dyn=dyn)
+    for j in range(5):
+        assert_close(fused[j], plain[j].float().cpu(), 2e-2, f"out[{j}]")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,C", [(1, 64), (9, 320), (130, 128), (64, 2560), (257, 4096)])
 @pytest.mark.parametrize("divisor,eps,gated", [(8.0, 1e-5, True), (1.0, 64e-5, True), (1.0, 1e-5, False)])

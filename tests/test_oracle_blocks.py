@@ -36,6 +36,26 @@ def test_mixes_at_the_ends_of_the_coefficient_range():
     assert torch.allclose(d, x + (xx - x) * (m + dyn[0]), atol=1e-14)
 
 
+def test_lora_mix_against_a_loop_of_matrix_vector_products():
+    B, T, C, D = 2, 5, 12, 4
+    x, s = _rand(B, T, C), _rand(B, C, seed=1)
+    maas = [torch.rand(1, 1, C, dtype=x.dtype, generator=torch.Generator().manual_seed(10 + j)) for j in range(5)]
+    act, w2 = _rand(B * T, 5, D, seed=2), _rand(5, D, C, seed=3)
+    outs = OB.lora_mix_v6(x, s, maas, act, w2)
+    xx = OB.token_shift(x, s)
+    for j in range(5):
+        for b in range(B):
+            for t in range(T):
+                dyn = w2[j].T @ act[b * T + t, j]                 # (C,): this token's, this mix's product
+                want = x[b, t] + (xx[b, t] - x[b, t]) * (maas[j].reshape(C) + dyn)
+                assert torch.allclose(outs[j][b, t], want, atol=1e-13)
+    # without the second factor the mixes are the plain ones
+    plain = OB.mix_v6(x, s, maas)
+    zero = OB.lora_mix_v6(x, s, maas, act, torch.zeros_like(w2))
+    for a, b_ in zip(plain, zero):
+        assert torch.equal(a, b_)
+
+
 def test_ln_x_gate_against_written_out_normalisation_and_layer_norm():
     H, C, N = 3, 192, 7
     y, gate = _rand(N, C), _rand(N, C, seed=1)
