@@ -1,13 +1,21 @@
 // RWKV-v4 WKV with (aa, bb, pp) state: one lane per (batch, channel) chain.
 //
-// The chain is serial in time, and a GPU holds few chains (B*C lanes: one or two
-// wavefronts per CU), so what sets the speed is how many bytes each lane keeps
-// in flight: blocks of 16 tokens of k, v (and gy) are fetched into registers
-// three blocks ahead of the one being consumed; consecutive lanes are consecutive
-// channels, so every load and store is a full coalesced row.  Per token the
-// arithmetic is kept short (one exponential per max-scaled pair, the bare
-// reciprocal instruction) and free of branches, so that the tokens of a block are
-// one straight-line stretch the scheduler can interleave.
+// The chain is serial in time, and a GPU holds few chains (B*C lanes), so two things set the speed: how many
+// bytes each lane keeps in flight, and how many instructions the ONE wavefront that walks a chain has to issue per
+// token.  For the first, blocks of 16 tokens of k, v (and gy) are fetched into registers several blocks ahead of the
+// one being consumed; consecutive lanes are consecutive channels, so every load and store is a full coalesced row.
+// For the second, only the recurrence itself stays with the walking wavefront; everything that can be formed from
+// a block's starting state alone is handed to other wavefronts of the workgroup, which work on different blocks at
+// the same time:
+//   forward   wavefront 0 advances (p, q, o) and leaves the state at the start of every 16-token block in LDS;
+//             wavefronts 1-3 take a block each (every third block) and form its 16 outputs from that state;
+//   backward  wavefront 0 replays a block from the forward's checkpoint and leaves what the reverse walk needs of
+//             its 16 tokens in LDS; wavefront 1 walks the block replayed just before backwards at the same time.
+//             (More replaying wavefronts, the 16-byte fetches of the forward, or two pairs per workgroup were all
+//             measured slower here: with the recurrence replayed the pass is bound by the instructions a compute
+//             unit issues, not by one wavefront's.)
+// Per token the arithmetic is kept short (one exponential per max-scaled pair, the bare reciprocal instruction) and
+// free of branches, so that the tokens of a block are one straight-line stretch the scheduler can interleave.
 //
 // State convention (RWKV-v4neo/cuda/wkv_cuda_bf16.cu:30-52): (p, q, o) with
 // p, q the decayed sums divided by e^{o}.  Backward carries the state gradient
@@ -17,8 +25,7 @@
 // Backward never stores per-token intermediates for the whole sequence (the
 // reference keeps three T-long arrays per lane): the forward sweep leaves a
 // 5-float checkpoint (p, q, o, dp/dw, dq/dw) every 16 tokens, and the backward
-// sweep replays one 16-token block at a time from its checkpoint (a second
-// wavefront walks the block replayed just before backwards at the same time).
+// sweep replays one 16-token block at a time from its checkpoint.
 #include "common.h"
 #include <type_traits>
 
@@ -65,76 +72,183 @@ __device__ __forceinline__ float v4_step(Chain &s, float w, float u, float kk, f
     return y;
 }
 
+// the recurrence alone: the same operations on (p, q, o, dp, dq) as v4_step, in the same order
+__device__ __forceinline__ void v4_advance(Chain &s, float w, float kk, float vv) {
+    const float wo = w + s.o;
+    const ExpPair d = exp_pair(wo, kk);
+    const float dh = d.first, dc = d.second;
+    s.dp = dh * (s.p + s.dp);
+    s.dq = dh * (s.q + s.dq);
+    s.p = fmaf(dh, s.p, dc * vv);
+    s.q = fmaf(dh, s.q, dc);
+    s.o = d.first_is_max ? wo : kk;
+}
+
+// A block of 16 tokens x 64 chains of one tensor on its way from memory to the lanes that own the chains.  A
+// wavefront can have 64 memory instructions in flight, so what it has in flight in bytes is set by the size of one:
+//   WIDE   16 bytes per lane: lane l fetches W = 16 / sizeof(T) consecutive chains of token l / (64/W) of every
+//          group of 64 / (64/W) tokens (a full 256- or 128-byte row segment per 64/W lanes); a block is 4 (fp32) or
+//          2 (bf16, fp16) instructions.  The pieces reach their owners through LDS: written as they came,
+//          [token][chain], read back one element per lane and token.  Needs C to be a multiple of W (a piece
+//          never straddles two batch rows) and 16-byte aligned tensors.
+//   narrow one element per lane and token: 16 instructions per block; any C.
+// Either way the block ends up in the LDS area handed in as well as in the caller's registers.
+template <class T, bool WIDE> struct V4In;
+template <class T> struct V4In<T, false> {
+    T val[CK];
+    __device__ __forceinline__ void fetch(const T *p, int /*chain0*/, int idx, int /*BC*/, int C, int Tlen, int t0, int /*lane*/) {
+        const int b = idx / C, c = idx % C;
+        const T *q = p + ((size_t)b * Tlen + t0) * C + c;
+        if (t0 + CK <= Tlen) {          // whole block inside the sequence: no per-token checks
+#pragma unroll
+            for (int i = 0; i < CK; i++, q += C) val[i] = *q;
+        } else {
+#pragma unroll
+            for (int i = 0; i < CK; i++, q += C) val[i] = t0 + i < Tlen ? *q : T{};
+        }
+    }
+    __device__ __forceinline__ void spread(T *stage, int lane, T (&out)[CK]) const {
+#pragma unroll
+        for (int i = 0; i < CK; i++) { out[i] = val[i]; stage[i * 64 + lane] = val[i]; }
+    }
+};
+template <class T> struct V4In<T, true> {
+    static constexpr int W = 16 / sizeof(T), LPR = 64 / W, ROWS = 64 / LPR, NLD = CK / ROWS;
+    typedef unsigned int piece_t __attribute__((ext_vector_type(4)));
+    piece_t piece[NLD];
+    // chain0: the wavefront's first chain (a multiple of 64); tokens past the end repeat the last one (never used)
+    __device__ __forceinline__ void fetch(const T *p, int chain0, int /*idx*/, int BC, int C, int Tlen, int t0, int lane) {
+        const int q = min(chain0 + (lane % LPR) * W, BC - W);
+        const T *row = p + (size_t)(q / C) * Tlen * C + q % C;
+#pragma unroll
+        for (int i = 0; i < NLD; i++)
+            piece[i] = *reinterpret_cast<const piece_t *>(row + (size_t)min(t0 + i * ROWS + lane / LPR, Tlen - 1) * C);
+    }
+    __device__ __forceinline__ void spread(T *stage, int lane, T (&out)[CK]) const {
+#pragma unroll
+        for (int i = 0; i < NLD; i++) *reinterpret_cast<piece_t *>(stage + (i * ROWS + lane / LPR) * 64 + (lane % LPR) * W) = piece[i];
+#pragma unroll
+        for (int i = 0; i < CK; i++) out[i] = stage[i * 64 + lane];
+    }
+};
+
 // Forward.  y == nullptr: only checkpoints / final state are produced.
 // ckpt layout: [block][5][B*C].
-template <class T>
-__global__ __launch_bounds__(64) void v4_forward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
+// Four wavefronts per 64 chains.  One walks the chain, V4_YW blocks (a round) between two workgroup barriers, and
+// leaves in LDS the state at the start of each block and the block's k and v; each of the other three forms the
+// outputs of one block of the round before from what it finds there (it reads nothing from memory).  The walking
+// wavefront's inputs wait in registers as they came, two rounds deep (converting at the fetch would make every load
+// wait for its data on the spot, and nothing would be in flight); register sets and LDS slots are fixed per use, two
+// rounds written out.
+constexpr int V4_YW = 3, V4_GROUPS = 2;
+template <class T, bool WIDE>
+__global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
         const float *__restrict__ time_first, const T *__restrict__ k, const T *__restrict__ v,
         const float *__restrict__ s_in, T *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt)
 {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= BC) return;
+    __shared__ float start_all[V4_GROUPS][2 * V4_YW][3][64];
+    // k and v of the blocks of two rounds, [token][chain]: left there by the walking wavefront on its way (it is also
+    // how the 16-byte pieces reach their owners), read by the wavefront that forms the block's outputs a round later
+    extern __shared__ __align__(16) unsigned char kv_raw[];          // v4_forward_lds<T>() bytes
+    typedef T KvBlock[CK * 64];
+    KvBlock (*kv_all)[2 * V4_YW][2] = reinterpret_cast<KvBlock (*)[2 * V4_YW][2]>(kv_raw);
+    // A workgroup is two groups of four wavefronts, 64 chains each.  The walking wavefront is the first of its four in
+    // group 0 and the second in group 1: wavefronts go to the four SIMDs in turn, and two walkers on one SIMD would
+    // share the one resource they are short of.
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), grp = wave >> 2, wl = wave & 3;
+    const int role = wl == grp ? 0 : (wl < grp ? wl + 1 : wl);       // 0: walks the chain; 1 + r: outputs of every third block
+    // (lanes and groups past the last chain stay, the 16-byte fetches being a wavefront's joint work and the barriers
+    // the workgroup's: they read the last chains' inputs and write nothing)
+    const int chain_grp = (blockIdx.x * V4_GROUPS + grp) * 64, chain0 = min(chain_grp, (BC - 1) / 64 * 64);
+    const int idx = min(chain0 + lane, BC - 1);
+    const bool live = chain_grp + lane < BC;
+    float (*start)[3][64] = start_all[grp];
     const int b = idx / C, c = idx % C;
     const float w = -__expf(time_decay[c]), u = time_first[c];
     const size_t base = (size_t)b * Tlen * C + c;
-    Chain s{0.f, 0.f, NEG_HUGE, 0.f, 0.f};
-    if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
+    const int nblk = (Tlen + CK - 1) / CK, nround = (nblk + V4_YW - 1) / V4_YW;
+    typedef V4In<T, WIDE> In;
 
-    // RING 16-token blocks of k, v per lane: one being consumed, the others in flight; indexed statically by unrolling
-    // (kept as they came: converting at the fetch would make every load wait for its data on the spot, and nothing
-    // would be in flight; the conversion happens where a value is used)
-    constexpr int RING = 4;
-    T bk[RING][CK], bv[RING][CK];
-    auto fetch = [&](int t0, T (&kk)[CK], T (&vv)[CK]) {
-        const T *kp = k + base + (size_t)t0 * C, *vp = v + base + (size_t)t0 * C;
-        if (t0 + CK <= Tlen) {          // whole block inside the sequence: no per-token checks
-#pragma unroll
-            for (int i = 0; i < CK; i++, kp += C, vp += C) { kk[i] = *kp; vv[i] = *vp; }
-        } else {
-#pragma unroll
-            for (int i = 0; i < CK; i++, kp += C, vp += C) {
-                const bool in = t0 + i < Tlen;
-                kk[i] = in ? *kp : T{};
-                vv[i] = in ? *vp : T{};
-            }
-        }
-    };
-#pragma unroll
-    for (int d = 0; d < RING; d++)
-        if (d * CK < Tlen) fetch(d * CK, bk[d], bv[d]);
-    for (int tb = 0, blk = 0; tb < Tlen; tb += RING * CK) {
-#pragma unroll
-        for (int d = 0; d < RING; d++, blk++) {
-            const int t0 = tb + d * CK;
-            if (t0 >= Tlen) break;
-            if (ckpt) {
+    if (role == 0) {
+        Chain s{0.f, 0.f, NEG_HUGE, 0.f, 0.f};
+        if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
+        // two rounds of blocks: one being consumed, one in flight (named, not an array: every use is a fixed register set)
+        static_assert(V4_YW == 3, "the rounds are written out for three blocks");
+        In k0, k1, k2, k3, k4, k5, v0, v1, v2, v3, v4, v5;
+        auto first = [&](int d, In &ik, In &iv) __attribute__((always_inline)) {
+            if (d < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, d * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, d * CK, lane); }
+        };
+        first(0, k0, v0); first(1, k1, v1); first(2, k2, v2); first(3, k3, v3); first(4, k4, v4); first(5, k5, v5);
+        auto block = [&](int blk, int slot, In &ik, In &iv) __attribute__((always_inline)) {
+            if (blk >= nblk) return;
+            start[slot][0][lane] = s.p; start[slot][1][lane] = s.q; start[slot][2][lane] = s.o;
+            if (ckpt && live) {
                 float *cp = ckpt + (size_t)blk * 5 * BC + idx;
                 cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
             }
-            const int cnt = min(CK, Tlen - t0);
-            // (y or no y, whole block or not: decided once per block, so that the 16 tokens are straight-line code)
-            auto tokens = [&](auto with_y, auto full) {
-                T *yp = y + base + (size_t)t0 * C;
+            T kk[CK], vv[CK];
+            ik.spread(kv_all[grp][slot][0], lane, kk);
+            iv.spread(kv_all[grp][slot][1], lane, vv);
+            const int nb = blk + 2 * V4_YW;
+            if (nb < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, nb * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, nb * CK, lane); }
+            const int t0 = blk * CK, cnt = min(CK, Tlen - t0);
+            if (cnt == CK) {
 #pragma unroll
-                for (int i = 0; i < CK; i++) {
-                    if (decltype(full)::value || i < cnt) {
-                        float iden, ec, hw, nm;
-                        const float yy = v4_step(s, w, u, to_float(bk[d][i]), to_float(bv[d][i]), iden, ec, hw, nm);
-                        if (decltype(with_y)::value) { stream1(yp, from_float<T>(yy)); yp += C; }
-                    }
-                }
-            };
-            if (y) {
-                if (cnt == CK) tokens(std::true_type{}, std::true_type{});
-                else tokens(std::true_type{}, std::false_type{});
+                for (int i = 0; i < CK; i++) v4_advance(s, w, to_float(kk[i]), to_float(vv[i]));
             } else {
-                if (cnt == CK) tokens(std::false_type{}, std::true_type{});
-                else tokens(std::false_type{}, std::false_type{});
+#pragma unroll
+                for (int i = 0; i < CK; i++)
+                    if (i < cnt) v4_advance(s, w, to_float(kk[i]), to_float(vv[i]));
             }
-            if (t0 + RING * CK < Tlen) fetch(t0 + RING * CK, bk[d], bv[d]);
+        };
+        for (int rd = 0; rd <= nround; rd += 2) {
+            block(rd * V4_YW, 0, k0, v0); block(rd * V4_YW + 1, 1, k1, v1); block(rd * V4_YW + 2, 2, k2, v2);
+            lds_barrier();
+            if (rd + 1 <= nround) {
+                block((rd + 1) * V4_YW, 3, k3, v3); block((rd + 1) * V4_YW + 1, 4, k4, v4); block((rd + 1) * V4_YW + 2, 5, k5, v5);
+                lds_barrier();
+            }
+        }
+        if (s_out && live) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
+    } else {
+        const int r = role - 1;
+        // the outputs of this wavefront's block of round pr (whose starting state and inputs wait in slot `slot`)
+        auto outputs = [&](int pr, int slot) __attribute__((always_inline)) {
+            const int blk = pr * V4_YW + r;
+            if (!y || pr < 0 || blk >= nblk) return;
+            Chain s{start[slot][0][lane], start[slot][1][lane], start[slot][2][lane], 0.f, 0.f};
+            const T *ks = kv_all[grp][slot][0], *vs = kv_all[grp][slot][1];
+            T kk[CK], vv[CK];
+#pragma unroll
+            for (int i = 0; i < CK; i++) { kk[i] = ks[i * 64 + lane]; vv[i] = vs[i * 64 + lane]; }
+            const int t0 = blk * CK, cnt = min(CK, Tlen - t0);
+            T *yp = y + base + (size_t)t0 * C;
+            if (cnt == CK) {
+#pragma unroll
+                for (int i = 0; i < CK; i++, yp += C) {
+                    float iden, ec, hw, nm;
+                    const float yy = v4_step(s, w, u, to_float(kk[i]), to_float(vv[i]), iden, ec, hw, nm);
+                    if (live) stream1(yp, from_float<T>(yy));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < CK; i++, yp += C)
+                    if (i < cnt) {
+                        float iden, ec, hw, nm;
+                        const float yy = v4_step(s, w, u, to_float(kk[i]), to_float(vv[i]), iden, ec, hw, nm);
+                        if (live) stream1(yp, from_float<T>(yy));
+                    }
+            }
+        };
+        for (int rd = 0; rd <= nround; rd += 2) {       // in round rd: the block of round rd-1
+            outputs(rd - 1, V4_YW + r);
+            lds_barrier();
+            if (rd + 1 <= nround) {
+                outputs(rd, r);
+                lds_barrier();
+            }
         }
     }
-    if (s_out) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
 }
 
 // Backward: two wavefronts per 64 chains.  Replaying a block from its checkpoint does not depend on the reverse
@@ -291,13 +405,35 @@ size_t v4_backward_workspace(int B, int Tlen, int C) {       // gw, gu partials 
     return 2 * (size_t)B * C * sizeof(float) + v4_checkpoint_bytes(B, Tlen, C);
 }
 
+// whether the 16-byte fetches apply: a piece of 16 / sizeof(T) chains must not straddle two batch rows, and the
+// tensors must be 16-byte aligned
+template <class T> static bool v4_wide(int C, std::initializer_list<const void *> tensors) {
+    if (C % (16 / (int)sizeof(T)) != 0) return false;
+    for (const void *p : tensors)
+        if (p && (reinterpret_cast<uintptr_t>(p) & 15u) != 0) return false;
+    return true;
+}
+
+template <class T> constexpr size_t v4_forward_lds() { return (size_t)V4_GROUPS * 2 * V4_YW * 2 * CK * 64 * sizeof(T); }
+
 template <class T>
 static hipError_t fwd(hipStream_t s, int B, int Tlen, int C, const float *td, const float *tf, const void *k,
                       const void *v, const float *s_in, void *y, float *s_out, float *ckpt) {
     const int BC = B * C;
+    static hipError_t lds_ok = [] {           // (more than the 64 KB a kernel gets by default, for fp32)
+        hipError_t e = hipFuncSetAttribute((const void *)v4_forward<T, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)v4_forward_lds<T>());
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)v4_forward<T, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)v4_forward_lds<T>());
+        return e;
+    }();
+    if (lds_ok != hipSuccess) return lds_ok;
     prof_begin(KID_V4_FORWARD, s);
-    hipLaunchKernelGGL((v4_forward<T>), dim3((BC + 63) / 64), dim3(64), 0, s, BC, Tlen, C, td, tf, (const T *)k,
-                       (const T *)v, s_in, (T *)y, s_out, ckpt);
+    const dim3 grid(((BC + 63) / 64 + V4_GROUPS - 1) / V4_GROUPS), block(64 * (1 + V4_YW) * V4_GROUPS);
+    if (v4_wide<T>(C, {k, v, y}))
+        hipLaunchKernelGGL((v4_forward<T, true>), grid, block, v4_forward_lds<T>(), s, BC, Tlen, C, td, tf, (const T *)k,
+                           (const T *)v, s_in, (T *)y, s_out, ckpt);
+    else
+        hipLaunchKernelGGL((v4_forward<T, false>), grid, block, v4_forward_lds<T>(), s, BC, Tlen, C, td, tf, (const T *)k,
+                           (const T *)v, s_in, (T *)y, s_out, ckpt);
     prof_end(KID_V4_FORWARD, s);
     return hipGetLastError();
 }
