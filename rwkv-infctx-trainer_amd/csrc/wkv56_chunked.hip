@@ -48,6 +48,9 @@ namespace chunked {
 // backward16: p5 top of the step (the prefetched inputs arrive), p6 results of the step before written out, p7 running
 //             sum inside the wavefronts + the wait for the others', p0 rest of prepare, p1 wait, p2 chains / builders,
 //             p3 wait, p4 block phase
+// summary_pass (all four wavefronts print): p0 prepare (with the wait for the prefetched inputs), p1 wait, p2 the next
+//             step's loads issued + the decay bookkeeping of wavefront 0, p3 the four blocks' MFMAs and the update of X,
+//             p4 wait
 #ifdef WKV_PHASE_TIMING
 #define PT_DECL long long pt_[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long pt_last_ = clock64();
 #define PT_MARK(i) { const long long now_ = clock64(); pt_[i] += now_ - pt_last_; pt_last_ = now_; }
