@@ -106,6 +106,19 @@ inline void prof_end(int id, hipStream_t s) {
     if (p.id == id && p.used < p.start.size()) { (void)hipEventRecord(p.stop[p.used], s); p.used++; }
 }
 
+// Set-up that belongs to a device (a kernel's raised LDS limit is a property of the code object loaded on that
+// device): runs `setup` the first time it is asked for the current device and hands back what it returned from then on.
+struct PerDevice {
+    hipError_t status[64];
+    PerDevice() { std::fill(status, status + 64, hipErrorNotReady); }
+    template <class F> hipError_t once(F setup) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return setup(); }
+        if (status[dev] == hipErrorNotReady) status[dev] = setup();
+        return status[dev];
+    }
+};
+
 // sum per-batch partials: in (B, n) -> out (n); fixed order, so repeatable
 static __global__ void sum_over_batch(int B, int n, const float *__restrict__ in, float *__restrict__ out) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;

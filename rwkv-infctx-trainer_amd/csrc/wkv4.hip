@@ -420,11 +420,12 @@ template <class T>
 static hipError_t fwd(hipStream_t s, int B, int Tlen, int C, const float *td, const float *tf, const void *k,
                       const void *v, const float *s_in, void *y, float *s_out, float *ckpt) {
     const int BC = B * C;
-    static hipError_t lds_ok = [] {           // (more than the 64 KB a kernel gets by default, for fp32)
+    static PerDevice lds_limit;
+    const hipError_t lds_ok = lds_limit.once([] {           // (more than the 64 KB a kernel gets by default, for fp32)
         hipError_t e = hipFuncSetAttribute((const void *)v4_forward<T, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)v4_forward_lds<T>());
         if (e == hipSuccess) e = hipFuncSetAttribute((const void *)v4_forward<T, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)v4_forward_lds<T>());
         return e;
-    }();
+    });
     if (lds_ok != hipSuccess) return lds_ok;
     prof_begin(KID_V4_FORWARD, s);
     const dim3 grid(((BC + 63) / 64 + V4_GROUPS - 1) / V4_GROUPS), block(64 * (1 + V4_YW) * V4_GROUPS);

@@ -1511,9 +1511,10 @@ size_t forward_workspace(int B, int Tlen, int H) { return layout(B, Tlen, H * HE
 size_t backward_workspace(int B, int Tlen, int C, int H) { return layout(B, Tlen, C, H, plan_groups(B * H, Tlen)).total; }
 
 // The 16-wavefront kernels use more LDS than a kernel gets by default.  Raising the limit is a property of the loaded
-// code object and is done once, from wkv_init() or from the first launch, whichever comes first.
+// code object and is done once per device, from wkv_init() or from the first launch there, whichever comes first.
 hipError_t init_kernels() {
-    static hipError_t status = [] {
+    static PerDevice done;
+    return done.once([] {
         auto allow = [](const void *kernel, size_t bytes) {
             return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         };
@@ -1524,8 +1525,7 @@ hipError_t init_kernels() {
         if (e == hipSuccess) e = allow((const void *)backward16<true, true>, sizeof(Bwd16Tiles));
         if (e == hipSuccess) e = allow((const void *)backward16<false, false>, sizeof(Bwd16Tiles));
         return e;
-    }();
-    return status;
+    });
 }
 
 // ckpt == nullptr: no checkpoints kept;  part == nullptr: the sequences run in one piece each
