@@ -63,7 +63,7 @@ def test_token_shift_mix(dtype, B, T, C, n, lerp, dyn):
 
 
 @pytest.mark.parametrize("B,T,C", [(1, 1, 32), (2, 7, 96), (3, 130, 64), (2, 128, 2560), (1, 200, 320), (2, 129, 32),
-                                   (1, 257, 128), (2, 16, 4096)])
+                                   (1, 257, 128), (2, 16, 4096), (3, 300, 72), (1, 65, 8), (2, 1, 200), (1, 513, 136)])
 def test_lora_shift_mix(B, T, C):
     """The five data-dependent mixes with the second LoRA product inside the kernel (bf16) against the oracle in fp32
     on the same rounded inputs: the five outputs and the gradients of x, the shift state, the five time_maa

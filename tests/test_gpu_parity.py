@@ -187,6 +187,37 @@ def test_v4_matches_oracle(dtype, T, with_state):
     assert_close(und(L["state"].grad), und(ref[4]), rt, "v4 gstate (undivided)")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,T,C", [(1, 50, 8), (2, 33, 100), (3, 17, 130), (1, 200, 64), (5, 97, 52), (2, 49, 256), (1, 96, 328)])
+def test_v4_shapes(dtype, B, T, C):
+    """Widths that take the 16-byte fetches of the forward (C a multiple of 4 for fp32, of 8 for the 16-bit types) and
+    widths that do not, chains that do not fill the last wavefront or the second group of the last workgroup, lengths
+    that end inside a block, inside a round of three blocks and on their boundaries: y, the state and every gradient."""
+    import rwkv_wkv_hip as W
+    wl = v4_case(B, T, C, dtype, seed=B + T + C, with_state=True)
+    t = wl.tensors
+    print(f"case v4 shapes {dtype} B={B} T={T} C={C}", flush=True)
+    f32 = lambda x: x.float()
+    y_ref, s_ref = O4.forward(t["time_decay"], f32(t["time_first"]), f32(t["k"]), f32(t["v"]), t["state"])
+    ref = O4.backward(t["time_decay"], f32(t["time_first"]), f32(t["k"]), f32(t["v"]), t["state"], f32(t["dy"]),
+                      t["dstate"])
+    g = {n: x.to(dev()) for n, x in t.items()}
+    L = {n: g[n].clone().requires_grad_(True) for n in ("time_decay", "time_first", "k", "v", "state")}
+    y, s = W.wkv_op(L["time_decay"], L["time_first"], L["k"], L["v"], L["state"])
+    torch.autograd.backward([y, s], [g["dy"], g["dstate"]])
+    torch.cuda.synchronize()
+    rt = RTOL[dtype]
+    assert y.dtype == dtype
+    assert_close(y, y_ref, rt, "v4 y")
+    und = lambda st: st[..., :2].float().cpu() * torch.exp(st[..., 2:3].float().cpu())
+    assert_close(und(s), und(s_ref), 1e-3, "v4 state (undivided sums)")
+    assert_close(L["time_decay"].grad, ref[0], rt, "v4 g_time_decay")
+    assert_close(L["time_first"].grad, ref[1], rt, "v4 g_time_first")
+    assert_close(L["k"].grad, ref[2], rt, "v4 gk")
+    assert_close(L["v"].grad, ref[3], rt, "v4 gv")
+    assert_close(und(L["state"].grad), und(ref[4]), rt, "v4 gstate (undivided)")
+
+
 def test_v4_backward_without_forward_checkpoints():
     """The C entry point rebuilds its checkpoints when none are passed."""
     import ctypes
