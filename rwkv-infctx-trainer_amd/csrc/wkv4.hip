@@ -134,12 +134,12 @@ template <class T> struct V4In<T, true> {
 
 // Forward.  y == nullptr: only checkpoints / final state are produced.
 // ckpt layout: [block][5][B*C].
-// Four wavefronts per 64 chains.  One walks the chain, V4_YW blocks (a round) between two workgroup barriers, and
+// Four wavefronts per 64 chains.  One walks the chain, V4_YW blocks (a lap) between two workgroup barriers, and
 // leaves in LDS the state at the start of each block and the block's k and v; each of the other three forms the
-// outputs of one block of the round before from what it finds there (it reads nothing from memory).  The walking
-// wavefront's inputs wait in registers as they came, two rounds deep (converting at the fetch would make every load
+// outputs of one block of the lap before from what it finds there (it reads nothing from memory).  The walking
+// wavefront's inputs wait in registers as they came, two laps deep (converting at the fetch would make every load
 // wait for its data on the spot, and nothing would be in flight); register sets and LDS slots are fixed per use, two
-// rounds written out.
+// laps written out.
 constexpr int V4_YW = 3, V4_GROUPS = 2;
 template <class T, bool WIDE>
 __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int BC, int Tlen, int C, const float *__restrict__ time_decay,
@@ -147,8 +147,8 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         const float *__restrict__ s_in, T *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt)
 {
     __shared__ float start_all[V4_GROUPS][2 * V4_YW][3][64];
-    // k and v of the blocks of two rounds, [token][chain]: left there by the walking wavefront on its way (it is also
-    // how the 16-byte pieces reach their owners), read by the wavefront that forms the block's outputs a round later
+    // k and v of the blocks of two laps, [token][chain]: left there by the walking wavefront on its way (it is also
+    // how the 16-byte pieces reach their owners), read by the wavefront that forms the block's outputs a lap later
     extern __shared__ __align__(16) unsigned char kv_raw[];          // v4_forward_lds<T>() bytes
     typedef T KvBlock[CK * 64];
     KvBlock (*kv_all)[2 * V4_YW][2] = reinterpret_cast<KvBlock (*)[2 * V4_YW][2]>(kv_raw);
@@ -166,14 +166,14 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
     const int b = idx / C, c = idx % C;
     const float w = -__expf(time_decay[c]), u = time_first[c];
     const size_t base = (size_t)b * Tlen * C + c;
-    const int nblk = (Tlen + CK - 1) / CK, nround = (nblk + V4_YW - 1) / V4_YW;
+    const int nblk = (Tlen + CK - 1) / CK, nlap = (nblk + V4_YW - 1) / V4_YW;
     typedef V4In<T, WIDE> In;
 
     if (role == 0) {
         Chain s{0.f, 0.f, NEG_HUGE, 0.f, 0.f};
         if (s_in) { s.p = s_in[idx * 3]; s.q = s_in[idx * 3 + 1]; s.o = s_in[idx * 3 + 2]; }
-        // two rounds of blocks: one being consumed, one in flight (named, not an array: every use is a fixed register set)
-        static_assert(V4_YW == 3, "the rounds are written out for three blocks");
+        // two laps of blocks: one being consumed, one in flight (named, not an array: every use is a fixed register set)
+        static_assert(V4_YW == 3, "the laps are written out for three blocks");
         In k0, k1, k2, k3, k4, k5, v0, v1, v2, v3, v4, v5;
         auto first = [&](int d, In &ik, In &iv) __attribute__((always_inline)) {
             if (d < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, d * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, d * CK, lane); }
@@ -201,10 +201,10 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
                     if (i < cnt) v4_advance(s, w, to_float(kk[i]), to_float(vv[i]));
             }
         };
-        for (int rd = 0; rd <= nround; rd += 2) {
+        for (int rd = 0; rd <= nlap; rd += 2) {
             block(rd * V4_YW, 0, k0, v0); block(rd * V4_YW + 1, 1, k1, v1); block(rd * V4_YW + 2, 2, k2, v2);
             lds_barrier();
-            if (rd + 1 <= nround) {
+            if (rd + 1 <= nlap) {
                 block((rd + 1) * V4_YW, 3, k3, v3); block((rd + 1) * V4_YW + 1, 4, k4, v4); block((rd + 1) * V4_YW + 2, 5, k5, v5);
                 lds_barrier();
             }
@@ -212,7 +212,7 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         if (s_out && live) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
     } else {
         const int r = role - 1;
-        // the outputs of this wavefront's block of round pr (whose starting state and inputs wait in slot `slot`)
+        // the outputs of this wavefront's block of lap pr (whose starting state and inputs wait in slot `slot`)
         auto outputs = [&](int pr, int slot) __attribute__((always_inline)) {
             const int blk = pr * V4_YW + r;
             if (!y || pr < 0 || blk >= nblk) return;
@@ -240,10 +240,10 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
                     }
             }
         };
-        for (int rd = 0; rd <= nround; rd += 2) {       // in round rd: the block of round rd-1
+        for (int rd = 0; rd <= nlap; rd += 2) {       // in lap rd: the block of lap rd-1
             outputs(rd - 1, V4_YW + r);
             lds_barrier();
-            if (rd + 1 <= nround) {
+            if (rd + 1 <= nlap) {
                 outputs(rd, r);
                 lds_barrier();
             }

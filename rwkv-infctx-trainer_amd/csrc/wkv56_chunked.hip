@@ -892,19 +892,26 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                         X[i] = role == 2 ? gp[x * HEAD + own] : gp[own * HEAD + x];
                     }
                 }
-            } else {
+            } else if (role == 1) {      // the summaries are read and chained once, by the value-major wavefronts
                 int ki[16], vi[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) { ki[i] = own; vi[i] = 16 * (i >> 2) + 4 * g + (i & 3); }
+                const float *pcs = gpart + (size_t)bh * nseg * m * PART, *ends = gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr;
+                chain_summaries<16, true>(X, ki, vi, pcs, (seg + 1) * m, (nseg - 1 - seg) * m, 1, ends);
+#pragma unroll
+                for (int i = 0; i < 16; i++) sm.q1[swz(own, vi[i])] = X[i];      // (the table is not in use yet)
+            }
+        }
+        if (seg != nseg - 1) {           // ... and handed to the other two roles through LDS, each in its own layout
+            lds_barrier();
+            if (role == 0 || role == 2) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int x = 16 * (i >> 2) + 4 * g + (i & 3);
-                    ki[i] = role == 2 ? x : own;
-                    vi[i] = role == 2 ? own : x;
+                    X[i] = role == 2 ? sm.q1[swz(x, own)] : sm.q1[swz(own, x)];
                 }
-                const float *pcs = gpart + (size_t)bh * nseg * m * PART, *ends = gs_out ? gs_out + (size_t)bh * HEAD * HEAD : nullptr;
-                if (role == 2) chain_summaries<16, false>(X, ki, vi, pcs, (seg + 1) * m, (nseg - 1 - seg) * m, 1, ends);
-                else chain_summaries<16, true>(X, ki, vi, pcs, (seg + 1) * m, (nseg - 1 - seg) * m, 1, ends);
-                have = true;
             }
+            have = role < 3;
         }
         if (have && (role == 1 || role == 2)) {
 #pragma unroll

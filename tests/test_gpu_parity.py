@@ -192,7 +192,7 @@ def test_v4_matches_oracle(dtype, T, with_state):
 def test_v4_shapes(dtype, B, T, C):
     """Widths that take the 16-byte fetches of the forward (C a multiple of 4 for fp32, of 8 for the 16-bit types) and
     widths that do not, chains that do not fill the last wavefront or the second group of the last workgroup, lengths
-    that end inside a block, inside a round of three blocks and on their boundaries: y, the state and every gradient."""
+    that end inside a block, inside a lap of three blocks and on their boundaries: y, the state and every gradient."""
     import rwkv_wkv_hip as W
     wl = v4_case(B, T, C, dtype, seed=B + T + C, with_state=True)
     t = wl.tensors
