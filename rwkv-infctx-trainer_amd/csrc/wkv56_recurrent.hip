@@ -28,6 +28,48 @@ __device__ __forceinline__ float group_sum(float x) {      // over the 4 lane gr
     return x;
 }
 
+// The 16 x 3 multiply-adds of one token on a lane's sixteen state elements, with the per-row (or per-column) factors
+// taken from the lane of this 16-lane row that holds them (a DPP operand: the broadcast costs no instruction).  The
+// sixteen lanes of a row need the same sixteen per-token values (r, k, w of the rows they share, or v, gy of the columns
+// they share); each lane reads ONE of them from LDS and the rest come across the row.  Read as four 16-byte pieces per
+// lane and tensor, these values were 12 to 20 KB of LDS traffic per wavefront and token, and the LDS port (128 bytes
+// per clock, shared by the wavefronts of a compute unit) was what bounded these kernels.
+//
+// Each token's instructions are ONE assembly statement: the compiler folds a DPP move into a multiply but not into a
+// fused multiply-add, and the hardware does not interlock a DPP read of a register that a vector instruction wrote
+// one or two slots earlier.  The statement opens with two wait states, and nothing can be placed inside it, so the
+// broadcast sources (inputs of the statement) are always old enough.  Within the statement the update of an element
+// is issued one element late, so that no instruction uses the result of the one before it.
+#define WKV_DPP(i) " row_newbcast:" #i " row_mask:0xf bank_mask:0xf\n\t"
+#define WKV_REP16(M) M(0) M(1) M(2) M(3) M(4) M(5) M(6) M(7) M(8) M(9) M(10) M(11) M(12) M(13) M(14) M(15)
+#define WKV_PIPE16(A, B) A(0) A(1) B(0) A(2) B(1) A(3) B(2) A(4) B(3) A(5) B(4) A(6) B(5) A(7) B(6) A(8) B(7) \
+                         A(9) B(8) A(10) B(9) A(11) B(10) A(12) B(11) A(13) B(12) A(14) B(13) A(15) B(14) B(15)
+#define WKV_S_OPERAND(i) [s##i] "+v"(S[i]),
+
+// acc += x[i] S[i];  S[i] = w[i] S[i] + k[i] v      (x, w, k broadcast from lane i of the row; v the lane's own)
+#define WKV_FWD_A(i) "v_fmac_f32_dpp %[acc], %[x], %[s" #i "]" WKV_DPP(i) "v_mul_f32_dpp %[s" #i "], %[w], %[s" #i "]" WKV_DPP(i)
+#define WKV_FWD_B(i) "v_fmac_f32_dpp %[s" #i "], %[k], %[v]" WKV_DPP(i)
+__device__ __forceinline__ void step_bcast_w(float (&S)[16], float &acc, float x, float w, float k, float v) {
+    asm("s_nop 1\n\t" WKV_PIPE16(WKV_FWD_A, WKV_FWD_B)
+        : WKV_REP16(WKV_S_OPERAND) [acc] "+v"(acc)
+        : [x] "v"(x), [w] "v"(w), [k] "v"(k), [v] "v"(v));
+}
+// acc += x[i] S[i];  S[i] = w S[i] + a[i] b         (x, a broadcast; w, b the lane's own)
+#define WKV_OWN_A(i) "v_fmac_f32_dpp %[acc], %[x], %[s" #i "]" WKV_DPP(i) "v_mul_f32 %[s" #i "], %[w], %[s" #i "]\n\t"
+#define WKV_OWN_B(i) "v_fmac_f32_dpp %[s" #i "], %[a], %[b]" WKV_DPP(i)
+__device__ __forceinline__ void step_own_w(float (&S)[16], float &acc, float x, float w, float a, float b) {
+    asm("s_nop 1\n\t" WKV_PIPE16(WKV_OWN_A, WKV_OWN_B)
+        : WKV_REP16(WKV_S_OPERAND) [acc] "+v"(acc)
+        : [x] "v"(x), [w] "v"(w), [a] "v"(a), [b] "v"(b));
+}
+__device__ __forceinline__ float token_sum(float x) {      // over the 16 lanes that stage one token
+    x += __shfl_xor(x, 1);
+    x += __shfl_xor(x, 2);
+    x += __shfl_xor(x, 4);
+    x += __shfl_xor(x, 8);
+    return x;
+}
+
 // ---------------------------------------------------------------- forward --
 template <class T, bool PER_TOKEN_W>
 __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
@@ -35,7 +77,9 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
         const float *__restrict__ wraw, const float *__restrict__ u,
         const float *__restrict__ s_in, T *__restrict__ y, float *__restrict__ s_out, int floor_decay)
 {
-    __shared__ __align__(16) float s_r[CH][HEAD], s_k[CH][HEAD], s_v[CH][HEAD], s_w[CH][HEAD], s_y[CH][HEAD];
+    __shared__ __align__(16) float s_r[CH][HEAD], s_k[CH][HEAD], s_v[CH][HEAD], s_w[CH][HEAD];
+    __shared__ __align__(16) float s_y[CH][4][HEAD];              // the four 16-row partial sums of each output
+    __shared__ float s_rho[CH];                                   // sum_i r u k of each staged token
 
     const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
@@ -43,14 +87,14 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int st = tid >> 4, sc = (tid & 15) * 4;            // staging: token st, channels sc..sc+3
 
-    float S[16], uu[16], wc[16];
+    const int shared_row = 16 * g + (lane & 15);            // the row whose r, k, w this lane reads for its 16-lane row
+    float S[16], us[4];
     const float *sp = s_in + (size_t)bh * HEAD * HEAD;
 #pragma unroll
-    for (int ii = 0; ii < 16; ii++) {
-        S[ii] = sp[(16 * g + ii) * HEAD + j];
-        uu[ii] = u[h * HEAD + 16 * g + ii];
-        wc[ii] = PER_TOKEN_W ? 0.f : __expf(log_decay(wraw[h * HEAD + 16 * g + ii], floor_decay));
-    }
+    for (int ii = 0; ii < 16; ii++) S[ii] = sp[(16 * g + ii) * HEAD + j];
+    const float w_const = PER_TOKEN_W ? 0.f : __expf(log_decay(wraw[h * HEAD + shared_row], floor_decay));
+#pragma unroll
+    for (int e = 0; e < 4; e++) us[e] = u[h * HEAD + sc + e];
 
     float pr[4], pk[4], pv[4], pw[4];
     auto fetch = [&](int t0) {
@@ -65,11 +109,15 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
         }
     };
     auto stage = [&]() {
+        float rho = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             s_r[st][sc + e] = pr[e]; s_k[st][sc + e] = pk[e]; s_v[st][sc + e] = pv[e];
             if (PER_TOKEN_W) s_w[st][sc + e] = __expf(log_decay(pw[e], floor_decay));
+            rho = fmaf(pr[e] * us[e], pk[e], rho);
         }
+        rho = token_sum(rho);
+        if (sc == 0) s_rho[st] = rho;
     };
 
     fetch(0);
@@ -78,32 +126,28 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
     for (int t0 = 0; t0 < Tlen; t0 += CH) {
         if (t0 + CH < Tlen) fetch(t0 + CH);
         const int nt = min(CH, Tlen - t0);      // the last block may be short
+        // The next token's LDS reads are issued ahead of this token's multiply-adds, and the four 16-row partial sums
+        // of an output go to LDS as they are: they are added (with the bonus term v rho) when the block's outputs
+        // are written out, so the token loop has no shuffle and no wait other than for its own operands.  A
+        // workgroup has one wavefront per SIMD; nothing else would hide those latencies.
+        float vj = s_v[0][j], r_sh = s_r[0][shared_row], k_sh = s_k[0][shared_row];
+        float w_sh = PER_TOKEN_W ? s_w[0][shared_row] : w_const;
         for (int t = 0; t < nt; t++) {
-            const float vj = s_v[t][j];
+            const int tn = t + 1 < CH ? t + 1 : t;
+            const float vj_n = s_v[tn][j], r_n = s_r[tn][shared_row], k_n = s_k[tn][shared_row];
+            const float w_n = PER_TOKEN_W ? s_w[tn][shared_row] : w_const;
             float acc = 0.f;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const float4 r4 = *reinterpret_cast<const float4 *>(&s_r[t][16 * g + 4 * q]);
-                const float4 k4 = *reinterpret_cast<const float4 *>(&s_k[t][16 * g + 4 * q]);
-                float4 w4;
-                if (PER_TOKEN_W) w4 = *reinterpret_cast<const float4 *>(&s_w[t][16 * g + 4 * q]);
-                else w4 = make_float4(wc[4 * q], wc[4 * q + 1], wc[4 * q + 2], wc[4 * q + 3]);
-                const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w},
-                            ww[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int ii = 4 * q + e;
-                    const float kv = kk[e] * vj;
-                    acc = fmaf(rr[e], fmaf(uu[ii], kv, S[ii]), acc);
-                    S[ii] = fmaf(ww[e], S[ii], kv);
-                }
-            }
-            acc = group_sum(acc);
-            if (g == 0) s_y[t][j] = acc;
+            step_bcast_w(S, acc, r_sh, w_sh, k_sh, vj);
+            s_y[t][g][j] = acc;
+            vj = vj_n; r_sh = r_n; k_sh = k_n; w_sh = w_n;
         }
         __syncthreads();
         if (t0 + st < Tlen) {
-            float o4[4] = {s_y[st][sc], s_y[st][sc + 1], s_y[st][sc + 2], s_y[st][sc + 3]};
+            float o4[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                o4[e] = fmaf(s_v[st][sc + e], s_rho[st],
+                             (s_y[st][0][sc + e] + s_y[st][1][sc + e]) + (s_y[st][2][sc + e] + s_y[st][3][sc + e]));
             store4(y + base + (size_t)(t0 + st) * C + sc, o4);
         }
         if (t0 + CH < Tlen) stage();
@@ -117,13 +161,19 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
 // --------------------------------------------------------------- backward --
 // Sweep 1 (forward in time, row-owned S):  gr_t, and q_t = r_t o gr_t kept in
 // fp32 for the decay-gradient sum.  Sweep 2 (backward in time, G held twice:
-// row-owned for gk, column-owned for gv):
-//     gk_t[i] = sum_j v_t[j] G[i][j] + u[i] r_t[i] (v_t.gy_t)
-//     gv_t[j] = sum_i k_t[i] ( G[i][j] + u[i] r_t[i] gy_t[j] )
+// row-owned for gk, column-owned for gv), with P_t = v_t.gy_t and rho_t = sum_i r_t[i] u[i] k_t[i]:
+//     gr_t[i] = sum_j gy_t[j] S[i][j] + u[i] k_t[i] P_t
+//     gk_t[i] = sum_j v_t[j] G[i][j] + u[i] r_t[i] P_t
+//     gv_t[j] = sum_i k_t[i] G[i][j] + gy_t[j] rho_t
 //     D_t[i]  = A[i] - k_t[i] sum_j v_t[j] G[i][j]          (= dL/d log w_t[i])
 //     A[i]   += q_t[i] - k_t[i] gk_t[i]
 //     G      <- w_t o G + r_t (x) gy_t
 // with A started from sum_j gS_out[i][j] S_out[i][j].
+//
+// The token loops only advance the states and leave the four 16-element partial sums of every contraction in LDS;
+// what follows from them (the sums, the bonus terms, the running sum A over the 16 tokens of a block) is done once per
+// block by all lanes: lane (g, row) takes tokens 4g..4g+3 of its row, and the A values at the starts of the four
+// token quarters come from three shuffles.
 template <class T, bool PER_TOKEN_W>
 __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         const T *__restrict__ r, const T *__restrict__ k, const T *__restrict__ v,
@@ -134,21 +184,28 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         float *__restrict__ qbuf, int floor_decay)
 {
     __shared__ __align__(16) float s_r[CH][HEAD], s_k[CH][HEAD], s_v[CH][HEAD], s_w[CH][HEAD], s_g[CH][HEAD],
-        s_l[CH][HEAD], s_q[CH][HEAD], o_a[CH][HEAD], o_b[CH][HEAD], o_c[CH][HEAD];
+        s_l[CH][HEAD], s_q[CH][HEAD];
+    __shared__ __align__(16) float p_a[CH][4][HEAD], p_b[CH][4][HEAD];   // partial sums [token][lane group][row or column]
+    __shared__ float s_p[CH], s_rho[CH];                                 // v.gy and sum r u k of each staged token
 
     const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int g = lane >> 4, own = 16 * wv + (lane & 15);    // own row i (row-owned) or own column j (column-owned)
+    const int shared = 16 * g + (lane & 15);                 // the column (row-owned) or row (column-owned) whose
+                                                             // per-token values this lane reads for its 16-lane row
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int st = tid >> 4, sc = (tid & 15) * 4;
 
     const float u_own = u[h * HEAD + own];
-    float l_own = 0.f, w_own = 1.f;
+    float l_own = 0.f, w_own = 1.f, w_shared = 1.f, us[4];
     bool floored_own = false;
     if (!PER_TOKEN_W) {
         l_own = log_decay(wraw[h * HEAD + own], floor_decay, &floored_own);
         w_own = __expf(l_own);
+        w_shared = __expf(log_decay(wraw[h * HEAD + shared], floor_decay));
     }
+#pragma unroll
+    for (int e = 0; e < 4; e++) us[e] = u[h * HEAD + sc + e];
 
     float pr[4], pk[4], pv[4], pw[4], pg[4], pq[4];
     auto fetch = [&](int t0, bool second) {
@@ -164,6 +221,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         }
     };
     auto stage = [&](bool second) {
+        float dot = 0.f, rho = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             s_r[st][sc + e] = pr[e]; s_k[st][sc + e] = pk[e]; s_v[st][sc + e] = pv[e]; s_g[st][sc + e] = pg[e];
@@ -174,7 +232,15 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
                 s_l[st][sc + e] = fl ? 0.f : l;          // factor that turns dL/d log w into dL/d raw
             }
             if (second) s_q[st][sc + e] = pq[e];
+            dot = fmaf(pv[e], pg[e], dot);
+            rho = fmaf(pr[e] * us[e], pk[e], rho);
         }
+        dot = token_sum(dot);
+        rho = token_sum(rho);
+        if (sc == 0) { s_p[st] = dot; s_rho[st] = rho; }
+    };
+    auto sum4 = [&](const float (&p)[CH][4][HEAD], int t, int x) {
+        return (p[t][0][x] + p[t][1][x]) + (p[t][2][x] + p[t][3][x]);
     };
 
     // ---------------- sweep 1: forward in time, S row-owned (row `own`, columns 16g..16g+15)
@@ -193,39 +259,36 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
     for (int t0 = 0; t0 < Tlen; t0 += CH) {
         if (t0 + CH < Tlen) fetch(t0 + CH, false);
         const int nt = min(CH, Tlen - t0);
+        float ki = s_k[0][own], wi = PER_TOKEN_W ? s_w[0][own] : w_own, v_sh = s_v[0][shared], g_sh = s_g[0][shared];
         for (int t = 0; t < nt; t++) {
-            const float ki = s_k[t][own], wi = PER_TOKEN_W ? s_w[t][own] : w_own;
-            const float uk = u_own * ki;
+            const int tn = t + 1 < CH ? t + 1 : t;
+            const float ki_n = s_k[tn][own], wi_n = PER_TOKEN_W ? s_w[tn][own] : w_own;
+            const float v_n = s_v[tn][shared], g_n = s_g[tn][shared];
             float acc = 0.f;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const float4 v4 = *reinterpret_cast<const float4 *>(&s_v[t][16 * g + 4 * q]);
-                const float4 g4 = *reinterpret_cast<const float4 *>(&s_g[t][16 * g + 4 * q]);
-                const float vv[4] = {v4.x, v4.y, v4.z, v4.w}, gg[4] = {g4.x, g4.y, g4.z, g4.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int jj = 4 * q + e;
-                    acc = fmaf(gg[e], fmaf(uk, vv[e], S[jj]), acc);
-                    S[jj] = fmaf(wi, S[jj], ki * vv[e]);
-                }
-            }
-            acc = group_sum(acc);
-            if (g == 0) { o_a[t][own] = acc; o_b[t][own] = acc * s_r[t][own]; }
+            step_own_w(S, acc, g_sh, wi, v_sh, ki);      // acc += gy_j S_ij;  S_ij = w_i S_ij + v_j k_i
+            p_a[t][g][own] = acc;
+            ki = ki_n; wi = wi_n; v_sh = v_n; g_sh = g_n;
         }
         __syncthreads();
         if (t0 + st < Tlen) {
             const size_t o = base + (size_t)(t0 + st) * C + sc;
-            float a4[4] = {o_a[st][sc], o_a[st][sc + 1], o_a[st][sc + 2], o_a[st][sc + 3]};
-            float b4[4] = {o_b[st][sc], o_b[st][sc + 1], o_b[st][sc + 2], o_b[st][sc + 3]};
+            float a4[4], b4[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                a4[e] = fmaf(us[e] * s_k[st][sc + e], s_p[st], sum4(p_a, st, sc + e));
+                b4[e] = a4[e] * s_r[st][sc + e];
+            }
             store4(gr + o, a4);
             store4(qbuf + o, b4);
         }
+        // no barrier: what the lines above read of the staged block and stage() overwrites is the lane's own four
+        // channels, or the token's scalar, which a lane of the same wavefront writes later in program order
         if (t0 + CH < Tlen) stage(false);
         __syncthreads();
     }
 
     // ---------------- boundary: G = gS_out in both ownerships, A = sum_j gS_out o S_out
-    float Gr[16], Gc[16], ucol[16], wcol[16];
+    float Gr[16], Gc[16];
     float A = 0.f;
     {
         const size_t so = (size_t)bh * HEAD * HEAD;
@@ -233,8 +296,6 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         for (int q = 0; q < 16; q++) {
             Gr[q] = gs_out ? gs_out[so + own * HEAD + 16 * g + q] : 0.f;
             Gc[q] = gs_out ? gs_out[so + (16 * g + q) * HEAD + own] : 0.f;
-            ucol[q] = u[h * HEAD + 16 * g + q];
-            wcol[q] = PER_TOKEN_W ? 0.f : __expf(log_decay(wraw[h * HEAD + 16 * g + q], floor_decay));
             A = fmaf(Gr[q], S[q], A);
         }
         A = group_sum(A);
@@ -252,63 +313,71 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
     __syncthreads();
     for (int t0 = last0; t0 >= 0; t0 -= CH) {
         if (t0 - CH >= 0) fetch(t0 - CH, true);
-        for (int t = min(CH, Tlen - t0) - 1; t >= 0; t--) {
-            // row-owned part (row i = own)
-            const float ri = s_r[t][own], ki = s_k[t][own], wi = PER_TOKEN_W ? s_w[t][own] : w_own;
-            float accG = 0.f, accP = 0.f;
-            // column-owned part (column j = own)
-            const float gyj = s_g[t][own];
-            float accV = 0.f;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const float4 v4 = *reinterpret_cast<const float4 *>(&s_v[t][16 * g + 4 * q]);
-                const float4 g4 = *reinterpret_cast<const float4 *>(&s_g[t][16 * g + 4 * q]);
-                const float4 r4 = *reinterpret_cast<const float4 *>(&s_r[t][16 * g + 4 * q]);
-                const float4 k4 = *reinterpret_cast<const float4 *>(&s_k[t][16 * g + 4 * q]);
-                float4 w4;
-                if (PER_TOKEN_W) w4 = *reinterpret_cast<const float4 *>(&s_w[t][16 * g + 4 * q]);
-                else w4 = make_float4(wcol[4 * q], wcol[4 * q + 1], wcol[4 * q + 2], wcol[4 * q + 3]);
-                const float vv[4] = {v4.x, v4.y, v4.z, v4.w}, gg[4] = {g4.x, g4.y, g4.z, g4.w},
-                            rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w},
-                            ww[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int x = 4 * q + e;
-                    accG = fmaf(vv[e], Gr[x], accG);
-                    accP = fmaf(vv[e], gg[e], accP);
-                    Gr[x] = fmaf(wi, Gr[x], ri * gg[e]);
-                    const float rg = rr[e] * gyj;
-                    accV = fmaf(kk[e], fmaf(ucol[x], rg, Gc[x]), accV);
-                    Gc[x] = fmaf(ww[e], Gc[x], rg);
-                }
+        const int nt = min(CH, Tlen - t0);
+        {
+            const int tf = nt - 1;
+            float ri = s_r[tf][own], wi = PER_TOKEN_W ? s_w[tf][own] : w_own, gyj = s_g[tf][own];
+            float v_sh = s_v[tf][shared], g_sh = s_g[tf][shared], r_sh = s_r[tf][shared], k_sh = s_k[tf][shared];
+            float w_sh = PER_TOKEN_W ? s_w[tf][shared] : w_shared;
+            for (int t = tf; t >= 0; t--) {
+                const int tn = t > 0 ? t - 1 : 0;
+                const float ri_n = s_r[tn][own], wi_n = PER_TOKEN_W ? s_w[tn][own] : w_own, gyj_n = s_g[tn][own];
+                const float v_n = s_v[tn][shared], g_n = s_g[tn][shared], r_n = s_r[tn][shared], k_n = s_k[tn][shared];
+                const float w_n = PER_TOKEN_W ? s_w[tn][shared] : w_shared;
+                float accG = 0.f, accV = 0.f;
+                step_own_w(Gr, accG, v_sh, wi, g_sh, ri);             // row i = own:    accG += v_j G_ij;  G_ij = w_i G_ij + gy_j r_i
+                step_bcast_w(Gc, accV, k_sh, w_sh, r_sh, gyj);        // column j = own: accV += k_i G_ij;  G_ij = w_i G_ij + r_i gy_j
+                p_a[t][g][own] = accG;
+                p_b[t][g][own] = accV;
+                ri = ri_n; wi = wi_n; gyj = gyj_n; v_sh = v_n; g_sh = g_n; r_sh = r_n; k_sh = k_n; w_sh = w_n;
             }
-            accG = group_sum(accG);
-            accP = group_sum(accP);
-            accV = group_sum(accV);
-            const float gki = fmaf(u_own * ri, accP, accG);
-            const float D = A - ki * accG;
-            A += s_q[t][own] - ki * gki;
-            gu_acc = fmaf(ri * ki, accP, gu_acc);
-            if (!PER_TOKEN_W) gw_acc += D;
-            if (g == 0) {
-                o_a[t][own] = gki;
-                o_b[t][own] = accV;
-                if (PER_TOKEN_W) o_c[t][own] = D * s_l[t][own];
+        }
+        __syncthreads();
+        {   // row `own`, tokens 4g+3 .. 4g: gk, and D from the running sum A (which runs from the last token down)
+            float c[4], kG[4], tot = 0.f;
+#pragma unroll
+            for (int e = 3; e >= 0; e--) {
+                const int t = 4 * g + e;
+                const float sumG = t < nt ? sum4(p_a, t, own) : 0.f;
+                const float ri = s_r[t][own], ki = s_k[t][own], rkP = ri * ki * s_p[t];
+                const float gki = fmaf(u_own * ri, s_p[t], sumG);
+                kG[e] = ki * sumG;
+                c[e] = s_q[t][own] - ki * gki;
+                tot += c[e];
+                gu_acc += rkP;
+                p_a[t][0][own] = gki;                    // read back below; this lane is the only one to touch (t, own)
             }
+            // A before token t = A + (c of all later tokens): later quarters, then later tokens of this quarter
+            const int low = lane & 15;
+            const float t1 = __shfl(tot, low + 16), t2 = __shfl(tot, low + 32), t3 = __shfl(tot, low + 48), t0q = __shfl(tot, low);
+            float run = A + (g < 1 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 3 ? t3 : 0.f);
+#pragma unroll
+            for (int e = 3; e >= 0; e--) {
+                const int t = 4 * g + e;
+                const float D = run - kG[e];
+                run += c[e];
+                if (PER_TOKEN_W) p_a[t][1][own] = D * s_l[t][own];
+                else if (t < nt) gw_acc += D;
+            }
+            A += (t0q + t1) + (t2 + t3);
         }
         __syncthreads();
         if (t0 + st < Tlen) {
             const size_t o = base + (size_t)(t0 + st) * C + sc;
-            float a4[4] = {o_a[st][sc], o_a[st][sc + 1], o_a[st][sc + 2], o_a[st][sc + 3]};
-            float b4[4] = {o_b[st][sc], o_b[st][sc + 1], o_b[st][sc + 2], o_b[st][sc + 3]};
+            float a4[4], b4[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                a4[e] = p_a[st][0][sc + e];
+                b4[e] = fmaf(s_g[st][sc + e], s_rho[st], sum4(p_b, st, sc + e));
+            }
             store4(gk + o, a4);
             store4(gv + o, b4);
             if (PER_TOKEN_W) {
-                float c4[4] = {o_c[st][sc], o_c[st][sc + 1], o_c[st][sc + 2], o_c[st][sc + 3]};
+                float c4[4] = {p_a[st][1][sc], p_a[st][1][sc + 1], p_a[st][1][sc + 2], p_a[st][1][sc + 3]};
                 store4(gw_tok + o, c4);
             }
         }
-        if (t0 - CH >= 0) stage(true);
+        if (t0 - CH >= 0) stage(true);           // no barrier needed, as in sweep 1
         __syncthreads();
     }
 
@@ -318,6 +387,8 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         for (int q = 0; q < 4; q++)
             *reinterpret_cast<float4 *>(gp + 4 * q) = make_float4(Gr[4 * q], Gr[4 * q + 1], Gr[4 * q + 2], Gr[4 * q + 3]);
     }
+    gu_acc = group_sum(gu_acc);
+    gw_acc = group_sum(gw_acc);
     if (g == 0) {
         gu_part[(size_t)bh * HEAD + own] = gu_acc;
         if (!PER_TOKEN_W) gw_part[(size_t)bh * HEAD + own] = floored_own ? 0.f : gw_acc * l_own;
