@@ -28,7 +28,8 @@ extern "C" {
 
 typedef enum {
     WKV_OK = 0,
-    WKV_ERR_DIMS = -1,        /* non-positive size, C != H*64, T too large for 32-bit indexing */
+    WKV_ERR_DIMS = -1,        /* non-positive size, C != H*64, T*C >= 2^30 (one sequence is addressed with 32-bit
+                                 byte offsets) or B*T*C >= 2^40 */
     WKV_ERR_NULL = -2,        /* a required pointer is NULL */
     WKV_ERR_DTYPE = -3,       /* dtype not one of wkv_dtype */
     WKV_ERR_ALIGN = -4,       /* a pointer is not 16-byte aligned */
@@ -138,7 +139,10 @@ int wkv6_forward_noalloc(void *stream, int B, int T, int C, int H, int dtype, un
 
 size_t wkv6_backward_workspace(int B, int T, int C, int H, int dtype, int algo);
 /* gstate_out may be NULL (no gradient arrives through the state handed out,
- * i.e. truncated BPTT); gstate_in may be NULL when it is not wanted. */
+ * i.e. truncated BPTT); gstate_in may be NULL when it is not wanted.  The two
+ * never overlap (WKV_ERR_ALIAS, for wkv5_backward as well): the state gradient
+ * of a head is shared by several workgroups, and some read gstate_out after
+ * others have written gstate_in. */
 int wkv6_backward(void *stream, int B, int T, int C, int H, int dtype, unsigned flags, int algo,
                   const void *r, const void *k, const void *v, const void *w, const float *u,
                   const float *state_in, const void *gy, const float *gstate_out,

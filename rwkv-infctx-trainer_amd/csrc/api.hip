@@ -21,6 +21,7 @@ int check_dims56(int B, int T, int C, int H, int dtype) {
     if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return WKV_ERR_DIMS;
     if (C != H * HEAD) return WKV_ERR_DIMS;
     if ((long long)B * T * C >= (1ll << 40)) return WKV_ERR_DIMS;
+    if ((long long)T * C >= (1ll << 30)) return WKV_ERR_DIMS;      // the kernels address a sequence with 32-bit byte offsets
     if (dtype < WKV_F32 || dtype > WKV_F16) return WKV_ERR_DTYPE;
     return WKV_OK;
 }
@@ -110,6 +111,12 @@ int backward56(bool per_token, void *stream, int B, int T, int C, int H, int dty
     if (workspace_bytes < (a == WKV_ALGO_CHUNKED ? chunked::backward_workspace(B, T, C, H)
                                                  : recurrent_backward_workspace(B, T, C)))
         return WKV_ERR_WORKSPACE;
+    if (gstate_in && gstate_out) {      // several workgroups share a head's state gradient: some read gstate_out after
+                                        // others have written gstate_in, so the two are never the same memory
+        const uintptr_t a0 = reinterpret_cast<uintptr_t>(gstate_in), b0 = reinterpret_cast<uintptr_t>(gstate_out);
+        const size_t bytes = (size_t)B * H * HEAD * HEAD * sizeof(float);
+        if (a0 < b0 + bytes && b0 < a0 + bytes) return WKV_ERR_ALIAS;
+    }
     if (a == WKV_ALGO_CHUNKED) {
         hipError_t e = chunked::backward_launch((hipStream_t)stream, per_token, w16, B, T, C, H, r, k, v, w, u, state_in, gy,
                                                 gstate_out, gr, gk, gv, gw, gu, gstate_in, workspace,
@@ -143,7 +150,7 @@ const char *wkv_strerror(int status) {
         case WKV_ERR_WORKSPACE: return "workspace too small";
         case WKV_ERR_LAUNCH: return "HIP launch failed";
         case WKV_ERR_ALGO: return "algorithm not available for this shape/dtype";
-        case WKV_ERR_ALIAS: return "state_out overlaps state_in (in place is possible only where no sequence is cut into time segments)";
+        case WKV_ERR_ALIAS: return "state_out overlaps state_in (in place is possible only where no sequence is cut into time segments), or gstate_in overlaps gstate_out (never possible)";
         default: return "unknown status";
     }
 }

@@ -39,6 +39,7 @@
 // (S_out = decay o S_in + delta), a small kernel chains the summaries into the state
 // at the start of every segment.  Backward does the same with the state gradient.
 #include "common.h"
+#include <type_traits>
 
 namespace wkv {
 namespace chunked {
@@ -146,21 +147,28 @@ __device__ __forceinline__ float group_sum4(float x) {      // over the 4 lane g
 // The raw decay of one token's four channels as it waits in registers between fetch and use: fp32, or bf16 as a
 // mixed-precision TimeMix hands it over (W16; converted where it is used, so the prefetch holds half the registers
 // and moves half the bytes).  For the time-invariant decay the same slot carries the constant log decay.
+// Element `o` of a sequence whose first element `p` points at, `p` being the same for all lanes: the byte offset is
+// formed in 32 bits, so the access takes the scalar base + 32-bit lane offset form and no lane holds a 64-bit address
+// (the launchers refuse a sequence of 2^30 elements or more per batch entry).
+template <class P> __device__ __forceinline__ P *seq_at(P *p, uint32_t o) {
+    using Byte = typename std::conditional<std::is_const<P>::value, const char, char>::type;
+    return reinterpret_cast<P *>(reinterpret_cast<Byte *>(p) + o * (uint32_t)sizeof(P));
+}
 template <bool W16> struct WReg;
 template <> struct WReg<false> {
     float4 v;
-    static __device__ __forceinline__ WReg load(const void *w, size_t o) {
-        return WReg{*reinterpret_cast<const float4 *>(static_cast<const float *>(w) + o)};
+    static __device__ __forceinline__ WReg load(const void *w, uint32_t o) {
+        return WReg{*reinterpret_cast<const float4 *>(seq_at(static_cast<const float *>(w), o))};
     }
     // The same as two 8-byte loads, for a value that stays in flight across a phase short of registers: a 16-byte load
     // wants four consecutive registers, which the allocator there gives only at the price of copies that wait for the
     // load on the spot.
-    static __device__ __forceinline__ WReg load_in_halves(const void *w, size_t o) {
+    static __device__ __forceinline__ WReg load_in_halves(const void *w, uint32_t o) {
         typedef float f2 __attribute__((ext_vector_type(2)));
-        size_t o2 = o + 2;
+        uint32_t o2 = o + 2;
         asm volatile("" : "+v"(o2));          // (opaque: the two loads are not seen to be adjacent, so they are not merged)
-        const f2 a = *reinterpret_cast<const f2 *>(static_cast<const float *>(w) + o);
-        const f2 b = *reinterpret_cast<const f2 *>(static_cast<const float *>(w) + o2);
+        const f2 a = *reinterpret_cast<const f2 *>(seq_at(static_cast<const float *>(w), o));
+        const f2 b = *reinterpret_cast<const f2 *>(seq_at(static_cast<const float *>(w), o2));
         return WReg{make_float4(a[0], a[1], b[0], b[1])};
     }
     static __device__ __forceinline__ WReg from(float4 x) { return WReg{x}; }
@@ -168,10 +176,10 @@ template <> struct WReg<false> {
 };
 template <> struct WReg<true> {
     uint2 v;
-    static __device__ __forceinline__ WReg load(const void *w, size_t o) {
-        return WReg{*reinterpret_cast<const uint2 *>(static_cast<const bf16 *>(w) + o)};
+    static __device__ __forceinline__ WReg load(const void *w, uint32_t o) {
+        return WReg{*reinterpret_cast<const uint2 *>(seq_at(static_cast<const bf16 *>(w), o))};
     }
-    static __device__ __forceinline__ WReg load_in_halves(const void *w, size_t o) { return load(w, o); }
+    static __device__ __forceinline__ WReg load_in_halves(const void *w, uint32_t o) { return load(w, o); }
     static __device__ __forceinline__ WReg from(float4 x) { return WReg{make_uint2(bf16_pack2(x.x, x.y), bf16_pack2(x.z, x.w))}; }
     __device__ __forceinline__ float4 f4() const { return make_float4(bf_lo(v.x), bf_hi(v.x), bf_lo(v.y), bf_hi(v.y)); }
 };
@@ -335,7 +343,11 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
     const int bh = bh0 + blockIdx.x / units, piece = (BACKWARD ? m : 0) + blockIdx.x % units, seg = piece / m, j = piece % m;
     const int b = bh / H, h = bh % H;
     const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
-    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    {       // the streams of this (batch, head): from here on every address is a 32-bit offset into its sequence
+        const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+        a_in += base; b_in += base;
+        if (PER_TOKEN_W) wraw = W16 ? (const void *)(static_cast<const bf16 *>(wraw) + base) : (const void *)(static_cast<const float *>(wraw) + base);
+    }
     const int nsb = (Tlen + SB - 1) / SB;
     const int sb0 = seg * sps + j * pps, sb1 = min(min(nsb, (seg + 1) * sps), sb0 + pps);
     const int nsteps = sb1 - sb0;
@@ -360,9 +372,9 @@ __global__ __launch_bounds__(NT_F) void summary_pass(int bh0, int Tlen, int C, i
         for (int x = 0; x < 4; x++) {
             const int t = sb * SB + tok0 + x;
             if (t < Tlen) {
-                const size_t o = base + (size_t)t * C + c4;
-                pa[x] = *reinterpret_cast<const uint2 *>(a_in + o);
-                pb[x] = *reinterpret_cast<const uint2 *>(b_in + o);
+                const uint32_t o = (uint32_t)t * C + c4;
+                pa[x] = *reinterpret_cast<const uint2 *>(seq_at(a_in, o));
+                pb[x] = *reinterpret_cast<const uint2 *>(seq_at(b_in, o));
                 pw[x] = PER_TOKEN_W ? WReg<W16>::load(wraw, o) : WReg<W16>::from(l_const);
             } else {
                 pa[x] = pb[x] = make_uint2(0u, 0u);
@@ -535,7 +547,11 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     const int q = w16 >> 2, wv = w16 & 3;          // block and quarter for preparing and finishing
     const bool chain = w16 < 8;                    // the other eight build the intra-block matrices: block wv, key half (w16 >> 2) & 1
     const int hk = w16 >> 2;                       // chain wavefronts: key half
-    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    {       // the streams of this (batch, head): from here on every address is a 32-bit offset into its sequence
+        const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+        r += base; k += base; v += base; y += base;
+        if (PER_TOKEN_W) wraw = W16 ? (const void *)(static_cast<const bf16 *>(wraw) + base) : (const void *)(static_cast<const float *>(wraw) + base);
+    }
     const int nsb = (Tlen + SB - 1) / SB;
     const int sb0 = seg * sps, sb1 = min(nsb, (seg + 1) * sps);
 
@@ -574,10 +590,10 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     auto fetch = [&](int sb, Row &x) __attribute__((always_inline)) {
         const int t = sb * SB + tok;
         if (t < Tlen) {
-            const size_t o = base + (size_t)t * C + c4;
-            x.r = *reinterpret_cast<const uint2 *>(r + o);
-            x.k = *reinterpret_cast<const uint2 *>(k + o);
-            x.v = *reinterpret_cast<const uint2 *>(v + o);
+            const uint32_t o = (uint32_t)t * C + c4;
+            x.r = *reinterpret_cast<const uint2 *>(seq_at(r, o));
+            x.k = *reinterpret_cast<const uint2 *>(seq_at(k, o));
+            x.v = *reinterpret_cast<const uint2 *>(seq_at(v, o));
             x.w = PER_TOKEN_W ? WReg<W16>::load(wraw, o) : WReg<W16>::from(l_const);
         } else {
             x.r = x.k = x.v = make_uint2(0u, 0u);
@@ -635,7 +651,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             const float uf[4] = {u4.x, u4.y, u4.z, u4.w};
             if (have_y) {      // y of the previous step waits in the rh tile: out as full rows, by the lanes that overwrite it next
                 const int t = (sb - 1) * SB + tok;
-                if (t < Tlen) store_row(y + base + (size_t)t * C + c4, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
+                if (t < Tlen) store_row(seq_at(y, (uint32_t)t * C + c4), *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
             }
             const bool whole = whole_step(sb);
             float rhv[4], khv[4], p = 0.f;
@@ -689,10 +705,11 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
                 split4(S[0], s0h, s0l);
                 split4(S[1], s1h, s1l);
                 const s4 r0 = frag(sm.rh, row, ca), r1 = frag(sm.rh, row, cb);
+                const s4 r0l = frag(sm.rhl, row, ca), r1l = frag(sm.rhl, row, cb);
                 f4 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = y0, y2 = y0;
+                y2 = mma2(r0l, r1l, s0h, s1h, y2);
                 y0 = mma2(r0, r1, s0h, s1h, y0);
                 y1 = mma2(r0, r1, s0l, s1l, y1);
-                y2 = mma2(frag(sm.rhl, row, ca), frag(sm.rhl, row, cb), s0h, s1h, y2);
                 // S <- e^{b} o S + (k e^{b-incl})^T v
                 const s4 v_op = frag_tr(sm.v, tro + (16 * blk) * LD + 16 * wv);
 #pragma unroll
@@ -711,18 +728,22 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             // A^T[s][t] = sum_i (k e^{b-incl})[s][i] (r e^{excl-b})[t][i]; lane gets s = 4g+e, t = n
             const int row = 16 * wv + n, kh2 = (w16 >> 2) & 1;
             f4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0;
+            const int ca = 32 * kh2 + 4 * g, cb = ca + 16;
+            // every LDS operand first, in one batch: a fetch issued where it is used costs the phase its latency
+            const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb), k0l = frag(sm.khl, row, ca), k1l = frag(sm.khl, row, cb);
+            const s4 ra = frag(sm.rh, row, ca), ral = frag(sm.rhl, row, ca), rb = frag(sm.rh, row, cb), rbl = frag(sm.rhl, row, cb);
+            const float4 ea = *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), eb = *reinterpret_cast<const float4 *>(&sm.ent[wv][cb]);
+            const float rho_t = kh2 ? 0.f : sm.rho[row];       // the diagonal goes with the first half
+            __builtin_amdgcn_sched_barrier(0);
             {
-                const int ca = 32 * kh2 + 4 * g, cb = ca + 16;
-                const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb);
                 s4 r0, r1, r0l, r1l;
-                scale_split(frag(sm.rh, row, ca), frag(sm.rhl, row, ca), *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), n == 0, r0, r0l);
-                scale_split(frag(sm.rh, row, cb), frag(sm.rhl, row, cb), *reinterpret_cast<const float4 *>(&sm.ent[wv][cb]), n == 0, r1, r1l);
+                scale_split(ra, ral, ea, n == 0, r0, r0l);
+                scale_split(rb, rbl, eb, n == 0, r1, r1l);
                 a0 = mma2(k0, k1, r0, r1, a0);
-                a1 = mma2(frag(sm.khl, row, ca), frag(sm.khl, row, cb), r0, r1, a1);
+                a1 = mma2(k0l, k1l, r0, r1, a1);
                 a2 = mma2(k0, k1, r0l, r1l, a2);
             }
             f4 at = a0 + (a1 + a2);
-            const float rho_t = kh2 ? 0.f : sm.rho[row];       // the diagonal goes with the first half
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int s_ = 4 * g + e;
@@ -760,7 +781,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
     }
     if (have_y) {
         const int t = (sb1 - 1) * SB + tok;
-        if (t < Tlen) store_row(y + base + (size_t)t * C + c4, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
+        if (t < Tlen) store_row(seq_at(y, (uint32_t)t * C + c4), *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
     }
     PT_PRINT("fwd16")
     if (chain && seg == nseg - 1) {
@@ -866,7 +887,14 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     const int bh = bh0 + blockIdx.x / nseg, seg = blockIdx.x % nseg, b = bh / H, h = bh % H;
     const int tid = threadIdx.x, w16 = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 4, n = lane & 15;
     const int role = w16 >> 2, q = role, wv = w16 & 3;      // chain role; block (for preparing and for the block phase); quarter
-    const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+    {       // the streams of this (batch, head): from here on every address is a 32-bit offset into its sequence
+        const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
+        r += base; k += base; v += base; gy += base; gr += base; gk += base; gv += base;
+        if (PER_TOKEN_W) {
+            wraw = W16 ? (const void *)(static_cast<const bf16 *>(wraw) + base) : (const void *)(static_cast<const float *>(wraw) + base);
+            gw_tok = W16 ? (void *)(static_cast<bf16 *>(gw_tok) + base) : (void *)(static_cast<float *>(gw_tok) + base);
+        }
+    }
     const int nsb = (Tlen + SB - 1) / SB;
     const int sb0 = seg * sps, sb1 = min(nsb, (seg + 1) * sps);
     const int own = 16 * wv + n;               // key (or, for the key-major gradient, value) channel of this lane
@@ -944,11 +972,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     auto fetch = [&](int sb, int tok, int c4) {       // (tok, c4 handed in: see WKV_LOCAL_LANE)
         const int t = sb * SB + tok;
         if (t < Tlen) {
-            const size_t o = base + (size_t)t * C + c4;
-            pr = *reinterpret_cast<const uint2 *>(r + o);
-            pk = *reinterpret_cast<const uint2 *>(k + o);
-            pv = *reinterpret_cast<const uint2 *>(v + o);
-            pg = *reinterpret_cast<const uint2 *>(gy + o);
+            const uint32_t o = (uint32_t)t * C + c4;
+            pr = *reinterpret_cast<const uint2 *>(seq_at(r, o));
+            pk = *reinterpret_cast<const uint2 *>(seq_at(k, o));
+            pv = *reinterpret_cast<const uint2 *>(seq_at(v, o));
+            pg = *reinterpret_cast<const uint2 *>(seq_at(gy, o));
             if (PER_TOKEN_W) pw = WReg<W16>::load(wraw, o);
         } else {
             pr = pk = pv = pg = make_uint2(0u, 0u);
@@ -959,11 +987,11 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     // are whole; a wait the compiler places after a conditional load is counted for the path without it
     auto fetch_whole = [&](int sb, int tok, int c4) {
         const int t = min(sb * SB + tok, Tlen - 1);
-        const size_t o = base + (size_t)t * C + c4;
-        pr = *reinterpret_cast<const uint2 *>(r + o);
-        pk = *reinterpret_cast<const uint2 *>(k + o);
-        pv = *reinterpret_cast<const uint2 *>(v + o);
-        pg = *reinterpret_cast<const uint2 *>(gy + o);
+        const uint32_t o = (uint32_t)t * C + c4;
+        pr = *reinterpret_cast<const uint2 *>(seq_at(r, o));
+        pk = *reinterpret_cast<const uint2 *>(seq_at(k, o));
+        pv = *reinterpret_cast<const uint2 *>(seq_at(v, o));
+        pg = *reinterpret_cast<const uint2 *>(seq_at(gy, o));
         if (PER_TOKEN_W) pw = WReg<W16>::load_in_halves(wraw, o);
     };
     const int lane0 = lane;
@@ -975,10 +1003,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         const int t = sb * SB + tok;
         if (!PER_TOKEN_W) {         // nothing per token to finish: gr, gk, gv only
             if (t < Tlen) {
-                const size_t o = base + (size_t)t * C + c4;
-                store_row(gr + o, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
-                store_row(gk + o, *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]));
-                store_row(gv + o, *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]));
+                const uint32_t o = (uint32_t)t * C + c4;
+                store_row(seq_at(gr, o), *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
+                store_row(seq_at(gk, o), *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]));
+                store_row(seq_at(gv, o), *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]));
             }
             return;
         }
@@ -999,10 +1027,10 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
         const float4 D = *reinterpret_cast<const float4 *>(&sm.incl[swz(tok, c4)]);
         A.x += D.x; A.y += D.y; A.z += D.z; A.w += D.w;
         if (t < Tlen) {
-            const size_t o = base + (size_t)t * C + c4;
-            store_row(gr + o, *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
-            store_row(gk + o, *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]));
-            store_row(gv + o, *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]));
+            const uint32_t o = (uint32_t)t * C + c4;
+            store_row(seq_at(gr, o), *reinterpret_cast<const uint2 *>(&sm.rh[tok * LD + c4]));
+            store_row(seq_at(gk, o), *reinterpret_cast<const uint2 *>(&sm.kh[tok * LD + c4]));
+            store_row(seq_at(gv, o), *reinterpret_cast<const uint2 *>(&sm.v[tok * LD + c4]));
             {                       // dL/dw_raw = dL/dlog w x log w (natural logarithm); nothing where the floor holds
                 const float4 l4 = *reinterpret_cast<const float4 *>(&sm.lw[swz(tok, c4)]);
                 const float lf[4] = {l4.x, l4.y, l4.z, l4.w};
@@ -1010,8 +1038,8 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
                 for (int c = 0; c < 4; c++) f[c] = (floor_decay && lf[c] <= LOG2_W_FLOOR) ? 0.f : lf[c] * LN2;
                 const float gw4[4] = {A.x * f[0], A.y * f[1], A.z * f[2], A.w * f[3]};
-                if (W16) store_row(static_cast<bf16 *>(gw_tok) + o, gw4);
-                else store_row(static_cast<float *>(gw_tok) + o, gw4);
+                if (W16) store_row(seq_at(static_cast<bf16 *>(gw_tok), o), gw4);
+                else store_row(seq_at(static_cast<float *>(gw_tok), o), gw4);
             }
         }
     };
@@ -1190,17 +1218,25 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
 #pragma unroll
             for (int qq = 3; qq >= 0; qq--) {
                 const int row = 16 * qq + n;
+                // The LDS operands of the block's products are fetched before the arithmetic on G starts: this wavefront
+                // is the longest of the phase and walks a dependent sequence, so a fetch issued where it is used costs
+                // the whole step its latency.
+                s4 kh_[4], kl_[4];
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    kh_[kk] = frag(sm.kh, row, 16 * kk + 4 * g);
+                    kl_[kk] = frag(sm.khl, row, 16 * kk + 4 * g);
+                }
+                __builtin_amdgcn_sched_barrier(0);
                 f4 g0 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kk = 0; kk < 4; kk += 2) {
-                    const int ca = 16 * kk + 4 * g, cb = ca + 16;
                     s4 g0h, g0l, g1h, g1l;
                     split4(G[kk], g0h, g0l);
                     split4(G[kk + 1], g1h, g1l);
-                    const s4 h0 = frag(sm.kh, row, ca), h1 = frag(sm.kh, row, cb);
-                    g0 = mma2(g0l, g1l, h0, h1, g0);       // (the gradient as the A operand: [value][token])
-                    g0 = mma2(g0h, g1h, frag(sm.khl, row, ca), frag(sm.khl, row, cb), g0);
-                    g0 = mma2(g0h, g1h, h0, h1, g0);
+                    g0 = mma2(g0l, g1l, kh_[kk], kh_[kk + 1], g0);       // (the gradient as the A operand: [value][token])
+                    g0 = mma2(g0h, g1h, kl_[kk], kl_[kk + 1], g0);
+                    g0 = mma2(g0h, g1h, kh_[kk], kh_[kk + 1], g0);
                 }
                 KG[qq] = g0;
                 if (qq == 3) sm.kg3[wv][lane] = make_float4(KG[3][0], KG[3][1], KG[3][2], KG[3][3]);
@@ -1216,8 +1252,12 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
             }
         } else {
             // ---------------- the masked matrices of block wv, once for everybody
+            // (the LDS operands of each matrix are fetched together and ahead of their use: the builders are, with the
+            // key-major chain, the longest wavefronts of the phase, and a fetch issued where it is used costs the whole
+            // step its latency)
             const int row = 16 * wv + n;
-            s4 gyf[4], vf[4];
+            s4 gyf[4], vf[4], rhf[4], rlf[4], khf[4], klf[4];
+            float4 en[4];
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) {
                 gyf[kk] = frag(sm.gy, row, 16 * kk + 4 * g);
@@ -1246,20 +1286,27 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
                 sm.pfr[wv][1][lane] = make_uint4(h0, h1, l0, l1);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // A~[t = 4g+e][s = n] = (r e^{excl-b})_t . (k e^{b-incl})_s
+            // A~[t = 4g+e][s = n] = (r e^{excl-b})_t . (k e^{b-incl})_s; its operands all at once
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                rhf[kk] = frag(sm.rh, row, 16 * kk + 4 * g);
+                rlf[kk] = frag(sm.rhl, row, 16 * kk + 4 * g);
+                khf[kk] = frag(sm.kh, row, 16 * kk + 4 * g);
+                klf[kk] = frag(sm.khl, row, 16 * kk + 4 * g);
+                en[kk] = *reinterpret_cast<const float4 *>(&sm.ent[wv][16 * kk + 4 * g]);
+            }
+            const float rho_s = sm.rho[row];
+            __builtin_amdgcn_sched_barrier(0);
             f4 at = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < 4; kk += 2) {
-                const int ca = 16 * kk + 4 * g, cb = ca + 16;
                 s4 r0, r1, r0l, r1l;
-                scale_split(frag(sm.rh, row, ca), frag(sm.rhl, row, ca), *reinterpret_cast<const float4 *>(&sm.ent[wv][ca]), n == 0, r0, r0l);
-                scale_split(frag(sm.rh, row, cb), frag(sm.rhl, row, cb), *reinterpret_cast<const float4 *>(&sm.ent[wv][cb]), n == 0, r1, r1l);
-                const s4 k0 = frag(sm.kh, row, ca), k1 = frag(sm.kh, row, cb);
-                at = mma2(r0l, r1l, k0, k1, at);
-                at = mma2(r0, r1, frag(sm.khl, row, ca), frag(sm.khl, row, cb), at);
-                at = mma2(r0, r1, k0, k1, at);
+                scale_split(rhf[kk], rlf[kk], en[kk], n == 0, r0, r0l);
+                scale_split(rhf[kk + 1], rlf[kk + 1], en[kk + 1], n == 0, r1, r1l);
+                at = mma2(r0l, r1l, khf[kk], khf[kk + 1], at);
+                at = mma2(r0, r1, klf[kk], klf[kk + 1], at);
+                at = mma2(r0, r1, khf[kk], khf[kk + 1], at);
             }
-            const float rho_s = sm.rho[row];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int x = 4 * g + e;

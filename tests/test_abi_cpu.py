@@ -48,6 +48,8 @@ def test_argument_checks_return_before_any_launch(L):
     assert L.wkv6_forward(null, 1, 8, 100, 2, 1, 0, 0, one, one, one, one, one, one, one, one, null, 0) == -1
     # non-positive T
     assert L.wkv5_forward(null, 1, 0, 64, 1, 1, 0, 0, one, one, one, one, one, one, one, one, null, 0) == -1
+    # a sequence too long for 32-bit byte offsets (T*C = 2^30)
+    assert L.wkv6_forward(null, 1, 1 << 18, 4096, 64, 1, 0, 0, one, one, one, one, one, one, one, one, null, 0) == -1
     # dtype out of range
     assert L.wkv6_forward(null, 1, 8, 64, 1, 7, 0, 0, one, one, one, one, one, one, one, one, null, 0) == -3
     # NULL r
@@ -63,6 +65,9 @@ def test_argument_checks_return_before_any_launch(L):
     assert need > 0
     args = [one] * 14
     assert L.wkv6_backward(null, 1, 8, 64, 1, 1, 1, 0, *args, one, need - 1) == -5   # flags = WKV_FLOOR_DECAY
+    # gstate_in overlapping gstate_out (arguments 8 and 14 of the 14 pointers), for either algorithm
+    assert L.wkv6_backward(null, 1, 8, 64, 1, 1, 1, 0, *args, one, need) == -8
+    assert L.wkv5_backward(null, 1, 8, 64, 1, 0, 1, 0, *args, one, L.wkv5_backward_workspace(1, 8, 64, 1, 0, 0)) == -8
     assert L.wkv4_forward(null, 0, 8, 64, 0, one, one, one, one, null, one, null, null) == -1
     assert L.wkv4_backward(null, 1, 8, 64, 0, *([one] * 13), one, 0) == -5
     assert L.wkv_cumsum_decay(null, 1, 100, 64, 16, 1, one, null, null, null, null, null) == -1
