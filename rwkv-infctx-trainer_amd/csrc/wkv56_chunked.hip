@@ -533,7 +533,9 @@ __device__ __forceinline__ void chain_summaries(float (&X)[N], const int (&ki)[N
     }
 }
 
-template <bool PER_TOKEN_W, bool W16>
+// ALL_WHOLE (time-invariant decay only): the sequence is a whole number of 64-token steps, so the general way of
+// a step with missing tokens is left out of the kernel, and with it the registers it keeps alive across the loop.
+template <bool PER_TOKEN_W, bool W16, bool ALL_WHOLE = false>
 __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const void *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
@@ -632,7 +634,7 @@ __global__ __launch_bounds__(NT_F16) void forward16(int bh0, int Tlen, int C, in
             *reinterpret_cast<float4 *>(&sm.ent[q][c4]) = make_float4(exp2_fast(-16.f * lcst[0]), exp2_fast(-16.f * lcst[1]), exp2_fast(-16.f * lcst[2]), exp2_fast(-16.f * lcst[3]));
         }
     }
-    auto whole_step = [&](int sb) { return !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
+    auto whole_step = [&](int sb) { return ALL_WHOLE ? true : !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
 #pragma unroll
     for (int c = 0; c < 4; c++) lc[c] = ic[c] = 0.f;
     if (!whole_step(sb0)) scan_ahead(rowA.w);
@@ -874,7 +876,7 @@ constexpr int NT_B16 = 1024;
               tok = 4 * w16 + g, tro = tr_lane_offset(lane, LD);                                              \
     (void)tro; (void)c4; (void)tok; (void)own;
 
-template <bool PER_TOKEN_W, bool W16>
+template <bool PER_TOKEN_W, bool W16, bool ALL_WHOLE = false>
 __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, int H, int nseg, int sps, int m,
         const bf16 *__restrict__ r, const bf16 *__restrict__ k, const bf16 *__restrict__ v,
         const void *__restrict__ wraw, const float *__restrict__ u, const bf16 *__restrict__ gy,
@@ -1052,7 +1054,7 @@ __global__ __launch_bounds__(NT_B16) void backward16(int bh0, int Tlen, int C, i
     // and overwrites the tables.
     float *const tab_r = sm.lw, *const tab_k = sm.lw + 16 * HEAD;
     bool tables_valid = false;
-    auto whole_step = [&](int sb) { return !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
+    auto whole_step = [&](int sb) { return ALL_WHOLE ? true : !PER_TOKEN_W && (sb + 1) * SB <= Tlen; };       // scalar
 
     fetch(sb1 - 1, tok, c4);
     if (tid < HEAD) sm.ub[tid] = u[h * HEAD + tid];
@@ -1575,9 +1577,11 @@ hipError_t init_kernels() {
         hipError_t e = allow((const void *)forward16<true, false>, sizeof(Fwd16Tiles));
         if (e == hipSuccess) e = allow((const void *)forward16<true, true>, sizeof(Fwd16Tiles));
         if (e == hipSuccess) e = allow((const void *)forward16<false, false>, sizeof(Fwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)forward16<false, false, true>, sizeof(Fwd16Tiles));
         if (e == hipSuccess) e = allow((const void *)backward16<true, false>, sizeof(Bwd16Tiles));
         if (e == hipSuccess) e = allow((const void *)backward16<true, true>, sizeof(Bwd16Tiles));
         if (e == hipSuccess) e = allow((const void *)backward16<false, false>, sizeof(Bwd16Tiles));
+        if (e == hipSuccess) e = allow((const void *)backward16<false, false, true>, sizeof(Bwd16Tiles));
         return e;
     });
 }
@@ -1618,6 +1622,9 @@ hipError_t forward_launch(hipStream_t s, bool per_token, bool w16, int B, int Tl
                                rr, kk, vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
         else if (mode == 1)
             hipLaunchKernelGGL((forward16<true, false>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
+                               rr, kk, vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
+        else if (Tlen % SB == 0)
+            hipLaunchKernelGGL((forward16<false, false, true>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
                                rr, kk, vv, w, u, s_in, (bf16 *)y, s_out, ckpt, part, floor_decay);
         else
             hipLaunchKernelGGL((forward16<false, false>), grid, block16, sizeof(Fwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps, x.m,
@@ -1688,6 +1695,10 @@ hipError_t backward_launch(hipStream_t s, bool per_token, bool w16, int B, int T
             hipLaunchKernelGGL((backward16<true, false>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps,
                                x.m, rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, gw, gw_part,
                                gu_part, gs_in, floor_decay);
+        else if (Tlen % SB == 0)
+            hipLaunchKernelGGL((backward16<false, false, true>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps,
+                               x.m, rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (void *)nullptr,
+                               gw_part, gu_part, gs_in, floor_decay);
         else
             hipLaunchKernelGGL((backward16<false, false>), grid, block16, sizeof(Bwd16Tiles), s, bh0, Tlen, C, H, x.nseg, x.sps,
                                x.m, rr, kk, vv, w, u, gg, gs_out, ckpt, gpart, (bf16 *)gr, (bf16 *)gk, (bf16 *)gv, (void *)nullptr,
