@@ -79,7 +79,7 @@ __device__ __forceinline__ void step_own_w(float (&S)[EL], float &acc, float x, 
 
 // Where a lane sits.  `own`: its column (column-owned) or row (row-owned), `ol` the same counted within the half;
 // `g8`: its group of eight rows (or columns); `shared`: the row (or column) whose per-token values it reads for its
-// 16-lane row; `slot`: where its partial sums go, after the lanes 32 apart have added theirs (pair_sum).
+// 16-lane row; `slot`: where its partial sums go, after the lanes 32 apart have added theirs (other_half).
 struct Place {
     int part, bh, wv, lane, gh, slot, ol, own, g8, shared;
     __device__ Place() {
@@ -461,7 +461,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
     }
     gu_acc = group_sum(gu_acc);
     gw_acc = group_sum(gw_acc);
-    if (scans && at.slot == 0) {
+    if (scans && at.slot == 0) {      // (two lanes of a row qualify: same value, same address)
         gu_part[(size_t)at.bh * HEAD + own] = gu_acc;
         if (!PER_TOKEN_W) gw_part[(size_t)at.bh * HEAD + own] = floored_own ? 0.f : gw_acc * l_own;
     }
