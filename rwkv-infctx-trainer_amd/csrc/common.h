@@ -128,4 +128,18 @@ static __global__ void sum_over_batch(int B, int n, const float *__restrict__ in
     out[i] = s;
 }
 
+// Compute units of the current device (256 on MI355X; also the answer when no device can be asked, as in a
+// workspace query made on a machine without one).
+inline int cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 256; }
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) { (void)hipGetLastError(); n = 256; }
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 }  // namespace wkv

@@ -1463,20 +1463,6 @@ size_t checkpoint_bytes(int B, int Tlen, int H) {
     return (size_t)B * H * ((Tlen + SB - 1) / SB + 1) * HEAD * HEAD * sizeof(float);     // one slot per step + the final state
 }
 
-// Compute units of the current device (256 on MI355X; also the answer when no device can be asked, as in a
-// workspace query made on a machine without one).
-static int cu_count() {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 256; }
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) { (void)hipGetLastError(); n = 256; }
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
 // How many time segments run in parallel for one (batch, head).  More segments mean
 // more workgroups (B*H*nseg) to spread over the compute units but also one more light pass
 // over (part of) the inputs; the estimate below counts CU rounds times steps

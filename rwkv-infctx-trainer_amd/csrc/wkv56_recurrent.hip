@@ -1,6 +1,7 @@
 // WKV5 / WKV6 per-token recurrence in fp32: the exact path (any T, any I/O dtype).
 //
-// Two workgroups of 256 lanes (4 wavefronts) per (batch, head), one per half of the head.  The 64x64 fp32 state of the
+// Described for its first form (the second, one workgroup per head with 16 elements per lane, is the same code with
+// other constants: `Shape`).  Two workgroups of 256 lanes (4 wavefronts) per (batch, head), one per half of the head.  The 64x64 fp32 state of the
 // head stays in VGPRs for the whole sequence: every lane keeps 8 elements, either "column-owned" (lane = one value
 // column j and a group of 8 key rows) or "row-owned" (lane = one key row i and a group of 8 value columns); a
 // workgroup has the 32 columns (or rows) of its half and all eight groups.  The contraction a step needs runs over the
@@ -26,8 +27,13 @@ namespace wkv {
 
 constexpr int CH = 16;            // tokens staged per step
 constexpr int NT = 256;           // lanes per workgroup
-constexpr int EL = 8;             // state elements per lane
-constexpr int HALF = HEAD / 2;    // columns (or rows) of a workgroup
+// EL = state elements per lane: 8 (two workgroups per head, each with 32 of its columns or rows: the form described
+// above) or 16 (one workgroup per head, four groups of 16: half the staging work per head, for batches whose heads
+// fill the compute units at least twice over anyway).  A workgroup has OWN = 4 EL columns (or rows).
+template <int EL> struct Shape {
+    static_assert(EL == 8 || EL == 16, "8 or 16 state elements per lane");
+    static constexpr int OWN = 4 * EL, PARTS = HEAD / OWN;
+};
 
 __device__ __forceinline__ float group_sum(float x) {      // over the 4 lane groups of 16
     x += __shfl_xor(x, 16);
@@ -57,66 +63,83 @@ __device__ __forceinline__ float token_sum(float x) {      // over the 16 lanes 
 // is issued one element late, so that no instruction uses the result of the one before it.
 #define WKV_DPP(i) " row_newbcast:" #i " row_mask:0xf bank_mask:0xf\n\t"
 #define WKV_REP8(M) M(0) M(1) M(2) M(3) M(4) M(5) M(6) M(7)
+#define WKV_REP16(M) WKV_REP8(M) M(8) M(9) M(10) M(11) M(12) M(13) M(14) M(15)
 #define WKV_PIPE8(A, B) A(0) A(1) B(0) A(2) B(1) A(3) B(2) A(4) B(3) A(5) B(4) A(6) B(5) A(7) B(6) B(7)
+#define WKV_PIPE16(A, B) A(0) A(1) B(0) A(2) B(1) A(3) B(2) A(4) B(3) A(5) B(4) A(6) B(5) A(7) B(6) A(8) B(7) \
+                         A(9) B(8) A(10) B(9) A(11) B(10) A(12) B(11) A(13) B(12) A(14) B(13) A(15) B(14) B(15)
 #define WKV_S_OPERAND(i) [s##i] "+v"(S[i]),
 
 // acc += x[i] S[i];  S[i] = w[i] S[i] + k[i] v      (x, w, k broadcast from lane i of the row; v the lane's own)
 #define WKV_FWD_A(i) "v_fmac_f32_dpp %[acc], %[x], %[s" #i "]" WKV_DPP(i) "v_mul_f32_dpp %[s" #i "], %[w], %[s" #i "]" WKV_DPP(i)
 #define WKV_FWD_B(i) "v_fmac_f32_dpp %[s" #i "], %[k], %[v]" WKV_DPP(i)
-__device__ __forceinline__ void step_bcast_w(float (&S)[EL], float &acc, float x, float w, float k, float v) {
+__device__ __forceinline__ void step_bcast_w(float (&S)[8], float &acc, float x, float w, float k, float v) {
     asm("s_nop 1\n\t" WKV_PIPE8(WKV_FWD_A, WKV_FWD_B)
         : WKV_REP8(WKV_S_OPERAND) [acc] "+v"(acc)
+        : [x] "v"(x), [w] "v"(w), [k] "v"(k), [v] "v"(v));
+}
+__device__ __forceinline__ void step_bcast_w(float (&S)[16], float &acc, float x, float w, float k, float v) {
+    asm("s_nop 1\n\t" WKV_PIPE16(WKV_FWD_A, WKV_FWD_B)
+        : WKV_REP16(WKV_S_OPERAND) [acc] "+v"(acc)
         : [x] "v"(x), [w] "v"(w), [k] "v"(k), [v] "v"(v));
 }
 // acc += x[i] S[i];  S[i] = w S[i] + a[i] b         (x, a broadcast; w, b the lane's own)
 #define WKV_OWN_A(i) "v_fmac_f32_dpp %[acc], %[x], %[s" #i "]" WKV_DPP(i) "v_mul_f32 %[s" #i "], %[w], %[s" #i "]\n\t"
 #define WKV_OWN_B(i) "v_fmac_f32_dpp %[s" #i "], %[a], %[b]" WKV_DPP(i)
-__device__ __forceinline__ void step_own_w(float (&S)[EL], float &acc, float x, float w, float a, float b) {
+__device__ __forceinline__ void step_own_w(float (&S)[8], float &acc, float x, float w, float a, float b) {
     asm("s_nop 1\n\t" WKV_PIPE8(WKV_OWN_A, WKV_OWN_B)
         : WKV_REP8(WKV_S_OPERAND) [acc] "+v"(acc)
         : [x] "v"(x), [w] "v"(w), [a] "v"(a), [b] "v"(b));
 }
+__device__ __forceinline__ void step_own_w(float (&S)[16], float &acc, float x, float w, float a, float b) {
+    asm("s_nop 1\n\t" WKV_PIPE16(WKV_OWN_A, WKV_OWN_B)
+        : WKV_REP16(WKV_S_OPERAND) [acc] "+v"(acc)
+        : [x] "v"(x), [w] "v"(w), [a] "v"(a), [b] "v"(b));
+}
 
-// Where a lane sits.  `own`: its column (column-owned) or row (row-owned), `ol` the same counted within the half;
-// `g8`: its group of eight rows (or columns); `shared`: the row (or column) whose per-token values it reads for its
-// 16-lane row; `slot`: where its partial sums go, after the lanes 32 apart have added theirs (other_half).
-struct Place {
-    int part, bh, wv, lane, gh, slot, ol, own, g8, shared;
+// Where a lane sits.  `own`: its column (column-owned) or row (row-owned), `ol` the same counted within the workgroup;
+// `grp`: its group of EL rows (or columns); `shared`: the row (or column) whose per-token values it reads for its
+// 16-lane row; `slot`: where its partial sums go (EL = 8: after the lanes 32 apart have added theirs, `paired`).
+template <int EL> struct Place {
+    int part, bh, wv, lane, gh, slot, ol, own, grp, shared;
     __device__ Place() {
-        part = blockIdx.x & 1; bh = blockIdx.x >> 1;
+        constexpr int PARTS = Shape<EL>::PARTS;
+        part = PARTS == 2 ? blockIdx.x & 1 : 0; bh = PARTS == 2 ? blockIdx.x >> 1 : blockIdx.x;
         wv = threadIdx.x >> 6; lane = threadIdx.x & 63;
-        gh = wv >> 1; slot = 2 * gh + ((lane >> 4) & 1);
-        ol = 16 * (wv & 1) + (lane & 15); own = HALF * part + ol;
-        g8 = 4 * gh + (lane >> 4); shared = EL * g8 + (lane & 7);
+        const int lg = lane >> 4;
+        gh = EL == 8 ? wv >> 1 : 0; slot = EL == 8 ? 2 * gh + (lg & 1) : lg;
+        ol = 16 * (EL == 8 ? wv & 1 : wv) + (lane & 15); own = Shape<EL>::OWN * part + ol;
+        grp = EL == 8 ? 4 * gh + lg : lg; shared = EL * grp + (lane & (EL - 1));
     }
 };
-using Partials = float[CH][4][HALF];
-__device__ __forceinline__ float other_half(float x) { return __shfl_xor(x, 32); }
-__device__ __forceinline__ float sum4(const Partials &p, int t, int x) {
+template <int EL> using Partials = float[CH][4][Shape<EL>::OWN];
+// what the lane 32 lanes away holds (EL = 8: the other row group of the pair that shares a slot; EL = 16: nothing to add)
+template <int EL> __device__ __forceinline__ float other_half(float x) { return EL == 8 ? __shfl_xor(x, 32) : 0.f; }
+template <class P> __device__ __forceinline__ float sum4(const P &p, int t, int x) {
     return (p[t][0][x] + p[t][1][x]) + (p[t][2][x] + p[t][3][x]);
 }
 
 // ---------------------------------------------------------------- forward --
-template <class T, bool PER_TOKEN_W>
+template <class T, bool PER_TOKEN_W, int EL>
 __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
         const T *__restrict__ r, const T *__restrict__ k, const T *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u,
         const float *__restrict__ s_in, T *__restrict__ y, float *__restrict__ s_out, int floor_decay)
 {
     __shared__ __align__(16) float s_r[CH][HEAD], s_k[CH][HEAD], s_v[CH][HEAD], s_w[CH][HEAD];
-    __shared__ __align__(16) Partials s_y;                        // partial sums of each output of this half
+    constexpr int OWN = Shape<EL>::OWN;
+    __shared__ __align__(16) Partials<EL> s_y;                    // partial sums of each output of this workgroup
     __shared__ float s_rho[CH];                                   // sum_i r u k of each staged token
 
-    const Place at;
+    const Place<EL> at;
     const int b = at.bh / H, h = at.bh % H, tid = threadIdx.x, j = at.own;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int st = tid >> 4, sc = (tid & 15) * 4;            // staging: token st, channels sc..sc+3
-    const bool writes = (sc >> 5) == at.part;                // ... and the lane writes them out if they are of this half
+    const bool writes = sc / OWN == at.part;                 // ... and the lane writes them out if they are of this workgroup
 
     float S[EL], us[4];
     const float *sp = s_in + (size_t)at.bh * HEAD * HEAD;
 #pragma unroll
-    for (int ii = 0; ii < EL; ii++) S[ii] = sp[(EL * at.g8 + ii) * HEAD + j];
+    for (int ii = 0; ii < EL; ii++) S[ii] = sp[(EL * at.grp + ii) * HEAD + j];
     const float w_const = PER_TOKEN_W ? 0.f : __expf(log_decay(wraw[h * HEAD + at.shared], floor_decay));
 #pragma unroll
     for (int e = 0; e < 4; e++) us[e] = u[h * HEAD + sc + e];
@@ -164,7 +187,7 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
         float done = 0.f;                        // the partial sum of the token before, not yet paired and stored
         auto token = [&](int t, const Tok &cur, Tok &nxt) {
             read(nxt, t + 1 < CH ? t + 1 : t);
-            const float there = other_half(done);
+            const float there = other_half<EL>(done);
             __builtin_amdgcn_sched_barrier(0);   // the reads and the shuffle are issued before the arithmetic, not after
             float acc = 0.f;
             step_bcast_w(S, acc, cur.r, cur.w, cur.k, cur.v);
@@ -177,12 +200,12 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
             token(t, ta, tb);
             if (t + 1 < nt) token(t + 1, tb, ta);
         }
-        s_y[nt - 1][at.slot][at.ol] = done + other_half(done);
+        s_y[nt - 1][at.slot][at.ol] = done + other_half<EL>(done);
         __syncthreads();
         if (writes) {
             float o4[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) o4[e] = fmaf(s_v[st][sc + e], s_rho[st], sum4(s_y, st, sc - HALF * at.part + e));
+            for (int e = 0; e < 4; e++) o4[e] = fmaf(s_v[st][sc + e], s_rho[st], sum4(s_y, st, sc - OWN * at.part + e));
             if (t0 + st < Tlen) store4(y + base + (size_t)(t0 + st) * C + sc, o4);
         }
         // no barrier: what the lines above read of the staged block and stage() overwrites is the lane's own four
@@ -192,7 +215,7 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
     }
     float *op = s_out + (size_t)at.bh * HEAD * HEAD;
 #pragma unroll
-    for (int ii = 0; ii < EL; ii++) op[(EL * at.g8 + ii) * HEAD + j] = S[ii];
+    for (int ii = 0; ii < EL; ii++) op[(EL * at.grp + ii) * HEAD + j] = S[ii];
 }
 
 // --------------------------------------------------------------- backward --
@@ -211,8 +234,9 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
 // them (the sums, the bonus terms, the running sum A over the 16 tokens of a block) is done once per block: lane
 // (g, row) of the first two wavefronts takes tokens 4g..4g+3 of its row, and the A values at the starts of the four
 // token quarters come from three shuffles.
-template <class T, bool PER_TOKEN_W>
-__global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
+// (EL = 8: four workgroups per compute unit, i.e. four wavefronts per SIMD, fit by LDS; the register budget is told so)
+template <class T, bool PER_TOKEN_W, int EL>
+__global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, int C, int H,
         const T *__restrict__ r, const T *__restrict__ k, const T *__restrict__ v,
         const float *__restrict__ wraw, const float *__restrict__ u, const float *__restrict__ s_in,
         const T *__restrict__ gy, const float *__restrict__ gs_out,
@@ -221,17 +245,18 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         float *__restrict__ qbuf, int floor_decay)
 {
     __shared__ __align__(16) float s_r[CH][HEAD], s_k[CH][HEAD], s_v[CH][HEAD], s_w[CH][HEAD], s_g[CH][HEAD],
-        s_l[CH][HALF];                                       // of the rows of this half
-    __shared__ __align__(16) Partials p_a, p_b;
+        s_l[CH][Shape<EL>::OWN];                             // of the rows of this workgroup
+    __shared__ __align__(16) Partials<EL> p_a, p_b;
     __shared__ float s_p[CH], s_rho[CH];                                 // v.gy and sum r u k of each staged token
 
-    const Place at;
+    const Place<EL> at;
     const int b = at.bh / H, h = at.bh % H, tid = threadIdx.x, own = at.own, ol = at.ol;
     const size_t base = (size_t)b * Tlen * C + (size_t)h * HEAD;
     const int st = tid >> 4, sc = (tid & 15) * 4;
-    const bool writes = (sc >> 5) == at.part;
-    const int wl = sc - HALF * at.part;                      // first of the lane's four channels within the half
-    const bool scans = at.gh == 0;                           // wavefronts 0 and 1: lane (lane group, ol)
+    constexpr int OWN = Shape<EL>::OWN;
+    const bool writes = sc / OWN == at.part;
+    const int wl = sc - OWN * at.part;                       // first of the lane's four channels within the workgroup's
+    const bool scans = at.gh == 0;                           // EL = 8: wavefronts 0 and 1; lane (lane group, ol)
 
     const float u_own = u[h * HEAD + own];
     float l_own = 0.f, w_own = 1.f, w_shared = 1.f, us[4];
@@ -284,10 +309,10 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         if (sc == 0) { s_p[st] = dot; s_rho[st] = rho; }
     };
 
-    // ---------------- sweep 1: forward in time, S row-owned (row `own`, columns 8 g8 .. 8 g8 + 7)
+    // ---------------- sweep 1: forward in time, S row-owned (row `own`, columns EL grp .. EL grp + EL - 1)
     float S[EL];
     {
-        const float *sp = s_in + (size_t)at.bh * HEAD * HEAD + own * HEAD + EL * at.g8;
+        const float *sp = s_in + (size_t)at.bh * HEAD * HEAD + own * HEAD + EL * at.grp;
 #pragma unroll
         for (int q = 0; q < EL / 4; q++) {
             const float4 x = *reinterpret_cast<const float4 *>(sp + 4 * q);
@@ -308,7 +333,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         float done = 0.f;
         auto token = [&](int t, const Tok &cur, Tok &nxt) {
             read(nxt, t + 1 < CH ? t + 1 : t);
-            const float there = other_half(done);
+            const float there = other_half<EL>(done);
             __builtin_amdgcn_sched_barrier(0);
             float acc = 0.f;
             step_own_w(S, acc, cur.g, cur.w, cur.v, cur.k);      // acc += gy_j S_ij;  S_ij = w_i S_ij + v_j k_i
@@ -321,7 +346,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
             token(t, ta, tb);
             if (t + 1 < nt) token(t + 1, tb, ta);
         }
-        p_a[nt - 1][at.slot][ol] = done + other_half(done);
+        p_a[nt - 1][at.slot][ol] = done + other_half<EL>(done);
         __syncthreads();
         if (writes) {
             float a4[4], b4[4];
@@ -350,11 +375,11 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
         float part = 0.f;
 #pragma unroll
         for (int q = 0; q < EL; q++) {
-            Gr[q] = gs_out ? gs_out[so + own * HEAD + EL * at.g8 + q] : 0.f;
-            Gc[q] = gs_out ? gs_out[so + (EL * at.g8 + q) * HEAD + own] : 0.f;
+            Gr[q] = gs_out ? gs_out[so + own * HEAD + EL * at.grp + q] : 0.f;
+            Gc[q] = gs_out ? gs_out[so + (EL * at.grp + q) * HEAD + own] : 0.f;
             part = fmaf(Gr[q], S[q], part);
         }
-        p_a[0][at.slot][ol] = part + other_half(part);
+        p_a[0][at.slot][ol] = part + other_half<EL>(part);
     }
     float gu_acc = 0.f, gw_acc = 0.f;
 
@@ -383,7 +408,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
             float doneG = 0.f, doneV = 0.f;
             auto token = [&](int t, const Tok &cur, Tok &nxt) {
                 read(nxt, t > 0 ? t - 1 : 0);
-                const float thereG = other_half(doneG), thereV = other_half(doneV);
+                const float thereG = other_half<EL>(doneG), thereV = other_half<EL>(doneV);
                 __builtin_amdgcn_sched_barrier(0);
                 float accG = 0.f, accV = 0.f;
                 step_own_w(Gr, accG, cur.vs, cur.w, cur.gs, cur.r);          // row i = own:    accG += v_j G_ij;  G_ij = w_i G_ij + gy_j r_i
@@ -400,8 +425,8 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
                 token(t, ta, tb);
                 if (t > 0) token(t - 1, tb, ta);
             }
-            p_a[0][at.slot][ol] = doneG + other_half(doneG);
-            p_b[0][at.slot][ol] = doneV + other_half(doneV);
+            p_a[0][at.slot][ol] = doneG + other_half<EL>(doneG);
+            p_b[0][at.slot][ol] = doneV + other_half<EL>(doneV);
         }
         __syncthreads();
         if (scans) {   // row `own`, tokens 4g+3 .. 4g: gk, and D from the running sum A (which runs from the last token down)
@@ -454,7 +479,7 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
     }
 
     if (gs_in) {
-        float *gp = gs_in + (size_t)at.bh * HEAD * HEAD + own * HEAD + EL * at.g8;
+        float *gp = gs_in + (size_t)at.bh * HEAD * HEAD + own * HEAD + EL * at.grp;
 #pragma unroll
         for (int q = 0; q < EL / 4; q++)
             *reinterpret_cast<float4 *>(gp + 4 * q) = make_float4(Gr[4 * q], Gr[4 * q + 1], Gr[4 * q + 2], Gr[4 * q + 3]);
@@ -468,39 +493,59 @@ __global__ __launch_bounds__(NT) void rec_backward(int Tlen, int C, int H,
 }
 
 // ------------------------------------------------------------- launchers --
-template <class T>
-static hipError_t launch_fwd(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
-                             const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
-                             int floor_decay) {
-    dim3 grid(2 * B * H), block(NT);
+// Eight elements per lane (two workgroups per head) where the finer grain evens out the load of the compute units;
+// sixteen where the heads fill them evenly anyway (a multiple of their number) or at least twice over: there the
+// staging work that two workgroups per head do twice costs more than the grain gains.  Forward + backward per token
+// on 256 compute units, ns, 8 / 16 elements: B*H = 128: 817 / 845; 256: 948 / 899; 320: 1180 / 1231; 384: 1219 / 1262;
+// 512: 1572 / 1355; 768: 2361 / 2025.  RWKV_WKV_REC_EL=8|16 overrides.
+static int elements_per_lane(int BH) {
+    static const int forced = [] { const char *e = getenv("RWKV_WKV_REC_EL"); return e ? atoi(e) : 0; }();
+    if (forced == 8 || forced == 16) return forced;
+    const int ncu = cu_count();
+    return (BH >= 2 * ncu || BH % ncu == 0) ? 16 : 8;
+}
+
+template <class T, int EL>
+static hipError_t launch_fwd_el(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
+                                const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
+                                int floor_decay) {
+    dim3 grid(Shape<EL>::PARTS * B * H), block(NT);
     prof_begin(KID_REC_FORWARD, s);
     if (per_token)
-        hipLaunchKernelGGL((rec_forward<T, true>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k, (const T *)v,
+        hipLaunchKernelGGL((rec_forward<T, true, EL>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k, (const T *)v,
                            w, u, s_in, (T *)y, s_out, floor_decay);
     else
-        hipLaunchKernelGGL((rec_forward<T, false>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
+        hipLaunchKernelGGL((rec_forward<T, false, EL>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
                            (const T *)v, w, u, s_in, (T *)y, s_out, floor_decay);
     prof_end(KID_REC_FORWARD, s);
     return hipGetLastError();
 }
-
 template <class T>
-static hipError_t launch_bwd(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
-                             const void *v, const float *w, const float *u, const float *s_in, const void *gy,
-                             const float *gs_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gs_in,
-                             float *ws, int floor_decay) {
+static hipError_t launch_fwd(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
+                             const void *v, const float *w, const float *u, const float *s_in, void *y, float *s_out,
+                             int floor_decay) {
+    return elements_per_lane(B * H) == 16
+               ? launch_fwd_el<T, 16>(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, y, s_out, floor_decay)
+               : launch_fwd_el<T, 8>(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, y, s_out, floor_decay);
+}
+
+template <class T, int EL>
+static hipError_t launch_bwd_el(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
+                                const void *v, const float *w, const float *u, const float *s_in, const void *gy,
+                                const float *gs_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gs_in,
+                                float *ws, int floor_decay) {
     // workspace: q (B,T,C) fp32 | gu partials (B,C) | gw partials (B,C)
     float *qbuf = ws;
     float *gu_part = qbuf + (size_t)B * Tlen * C;
     float *gw_part = gu_part + (size_t)B * C;
-    dim3 grid(2 * B * H), block(NT);
+    dim3 grid(Shape<EL>::PARTS * B * H), block(NT);
     prof_begin(KID_REC_BACKWARD, s);
     if (per_token)
-        hipLaunchKernelGGL((rec_backward<T, true>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
+        hipLaunchKernelGGL((rec_backward<T, true, EL>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
                            (const T *)v, w, u, s_in, (const T *)gy, gs_out, (T *)gr, (T *)gk, (T *)gv, gw, gw_part,
                            gu_part, gs_in, qbuf, floor_decay);
     else
-        hipLaunchKernelGGL((rec_backward<T, false>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
+        hipLaunchKernelGGL((rec_backward<T, false, EL>), grid, block, 0, s, Tlen, C, H, (const T *)r, (const T *)k,
                            (const T *)v, w, u, s_in, (const T *)gy, gs_out, (T *)gr, (T *)gk, (T *)gv, nullptr, gw_part,
                            gu_part, gs_in, qbuf, floor_decay);
     prof_end(KID_REC_BACKWARD, s);
@@ -509,6 +554,15 @@ static hipError_t launch_bwd(hipStream_t s, bool per_token, int B, int Tlen, int
     hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gu_part, gu);
     if (!per_token) hipLaunchKernelGGL(sum_over_batch, dim3((C + 255) / 256), dim3(256), 0, s, B, C, gw_part, gw);
     return hipGetLastError();
+}
+template <class T>
+static hipError_t launch_bwd(hipStream_t s, bool per_token, int B, int Tlen, int C, int H, const void *r, const void *k,
+                             const void *v, const float *w, const float *u, const float *s_in, const void *gy,
+                             const float *gs_out, void *gr, void *gk, void *gv, float *gw, float *gu, float *gs_in,
+                             float *ws, int floor_decay) {
+    return elements_per_lane(B * H) == 16
+               ? launch_bwd_el<T, 16>(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, gy, gs_out, gr, gk, gv, gw, gu, gs_in, ws, floor_decay)
+               : launch_bwd_el<T, 8>(s, per_token, B, Tlen, C, H, r, k, v, w, u, s_in, gy, gs_out, gr, gk, gv, gw, gu, gs_in, ws, floor_decay);
 }
 
 size_t recurrent_backward_workspace(int B, int Tlen, int C) {
