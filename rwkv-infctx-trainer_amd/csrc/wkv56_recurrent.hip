@@ -144,22 +144,24 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
 #pragma unroll
     for (int e = 0; e < 4; e++) us[e] = u[h * HEAD + sc + e];
 
+    // The fetch has no branch (the token is clamped into the sequence and what came for a token outside it is
+    // replaced where it is staged): loads and stores share one counter, and after a conditional load, or before a
+    // register a load may still be writing is set by hand, the compiler waits for everything outstanding, which here
+    // would be the stores of the block before.
     float pr[4], pk[4], pv[4], pw[4];
+    bool p_in = false;
     auto fetch = [&](int t0) {
         const int t = t0 + st;
-        if (t < Tlen) {
-            const size_t o = base + (size_t)t * C + sc;
-            load4(r + o, pr); load4(k + o, pk); load4(v + o, pv);
-            if (PER_TOKEN_W) load4(wraw + o, pw);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) { pr[e] = pk[e] = pv[e] = 0.f; pw[e] = -1e30f; }   // decay 1, no update
-        }
+        p_in = t < Tlen;
+        const size_t o = base + (size_t)min(t, Tlen - 1) * C + sc;
+        load4(r + o, pr); load4(k + o, pk); load4(v + o, pv);
+        if (PER_TOKEN_W) load4(wraw + o, pw);
     };
     auto stage = [&]() {
         float rho = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
+            if (!p_in) { pr[e] = pk[e] = pv[e] = 0.f; pw[e] = -1e30f; }   // decay 1, no update
             s_r[st][sc + e] = pr[e]; s_k[st][sc + e] = pk[e]; s_v[st][sc + e] = pv[e];
             if (PER_TOKEN_W) s_w[st][sc + e] = __expf(log_decay(pw[e], floor_decay));
             rho = fmaf(pr[e] * us[e], pk[e], rho);
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
     stage();
     __syncthreads();
     for (int t0 = 0; t0 < Tlen; t0 += CH) {
-        if (t0 + CH < Tlen) fetch(t0 + CH);
+        fetch(t0 + CH);                          // (past the end: a clamped fetch that nobody stages)
         const int nt = min(CH, Tlen - t0);      // the last block may be short
         // The next token's LDS reads are issued ahead of this token's multiply-adds, and the partial sums of an
         // output go to LDS as they are: they are added up (with the bonus term v rho) when the block's outputs are
@@ -202,15 +204,18 @@ __global__ __launch_bounds__(NT) void rec_forward(int Tlen, int C, int H,
         }
         s_y[nt - 1][at.slot][at.ol] = done + other_half<EL>(done);
         __syncthreads();
+        float o4[4];
         if (writes) {
-            float o4[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) o4[e] = fmaf(s_v[st][sc + e], s_rho[st], sum4(s_y, st, sc - OWN * at.part + e));
-            if (t0 + st < Tlen) store4(y + base + (size_t)(t0 + st) * C + sc, o4);
         }
         // no barrier: what the lines above read of the staged block and stage() overwrites is the lane's own four
         // channels, or the token's scalar, which a lane of the same wavefront writes later in program order
-        if (t0 + CH < Tlen) stage();
+        stage();                                 // (after the last block: zeros, unused; unconditional so that no load is left
+                                                 // outstanding on any path around the loop)
+        // The stores come after stage(): loads and stores share one counter, stage() waits for the prefetched block
+        // with a wait for everything outstanding, and a store issued before it would be waited for to the end.
+        if (writes && t0 + st < Tlen) store4(y + base + (size_t)(t0 + st) * C + sc, o4);
         __syncthreads();
     }
     float *op = s_out + (size_t)at.bh * HEAD * HEAD;
@@ -271,21 +276,20 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
 
     float pr[4], pk[4], pv[4], pw[4], pg[4];
     float pq[4], q_own[4];                                   // q of the lane's row at the four tokens it scans: in flight, current
+    bool p_in = false;                                       // (a fetch without branches, as in the forward)
+    int p_t0 = 0;
     auto fetch = [&](int t0, bool second) {
         const int t = t0 + st;
-        if (t >= 0 && t < Tlen) {
-            const size_t o = base + (size_t)t * C + sc;
-            load4(r + o, pr); load4(k + o, pk); load4(v + o, pv); load4(gy + o, pg);
-            if (PER_TOKEN_W) load4(wraw + o, pw);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) { pr[e] = pk[e] = pv[e] = pg[e] = 0.f; pw[e] = -1e30f; }
-        }
+        p_t0 = t0;
+        p_in = t >= 0 && t < Tlen;
+        const size_t o = base + (size_t)min(max(t, 0), Tlen - 1) * C + sc;
+        load4(r + o, pr); load4(k + o, pk); load4(v + o, pv); load4(gy + o, pg);
+        if (PER_TOKEN_W) load4(wraw + o, pw);
         if (second && scans) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int tq = t0 + 4 * (at.lane >> 4) + e;
-                pq[e] = tq >= 0 && tq < Tlen ? qbuf[base + (size_t)tq * C + own] : 0.f;
+                pq[e] = qbuf[base + (size_t)min(max(tq, 0), Tlen - 1) * C + own];
             }
         }
     };
@@ -293,6 +297,7 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
         float dot = 0.f, rho = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
+            if (!p_in) { pr[e] = pk[e] = pv[e] = pg[e] = 0.f; pw[e] = -1e30f; }
             s_r[st][sc + e] = pr[e]; s_k[st][sc + e] = pk[e]; s_v[st][sc + e] = pv[e]; s_g[st][sc + e] = pg[e];
             if (PER_TOKEN_W) {
                 bool fl;
@@ -300,7 +305,10 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
                 s_w[st][sc + e] = __expf(l);
                 if (writes) s_l[st][wl + e] = fl ? 0.f : l;      // factor that turns dL/d log w into dL/d raw
             }
-            if (second) q_own[e] = pq[e];
+            if (second) {
+                const int tq = p_t0 + 4 * (at.lane >> 4) + e;
+                q_own[e] = tq >= 0 && tq < Tlen ? pq[e] : 0.f;
+            }
             dot = fmaf(pv[e], pg[e], dot);
             rho = fmaf(pr[e] * us[e], pk[e], rho);
         }
@@ -323,7 +331,7 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
     stage(false);
     __syncthreads();
     for (int t0 = 0; t0 < Tlen; t0 += CH) {
-        if (t0 + CH < Tlen) fetch(t0 + CH, false);
+        fetch(t0 + CH, false);                   // (past the end: a clamped fetch that nobody stages)
         const int nt = min(CH, Tlen - t0);
         struct Tok { float k, w, v, g; };        // k, w of the lane's row; v, gy of the column it reads for its 16-lane row
         auto read = [&](Tok &x, int t) {
@@ -348,22 +356,22 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
         }
         p_a[nt - 1][at.slot][ol] = done + other_half<EL>(done);
         __syncthreads();
+        float a4[4], b4[4];
         if (writes) {
-            float a4[4], b4[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 a4[e] = fmaf(us[e] * s_k[st][sc + e], s_p[st], sum4(p_a, st, wl + e));
                 b4[e] = a4[e] * s_r[st][sc + e];
             }
-            if (t0 + st < Tlen) {
-                const size_t o = base + (size_t)(t0 + st) * C + sc;
-                store4(gr + o, a4);
-                store4(qbuf + o, b4);
-            }
         }
         // no barrier: what the lines above read of the staged block and stage() overwrites is the lane's own four
         // channels, or the token's scalar, which a lane of the same wavefront writes later in program order
-        if (t0 + CH < Tlen) stage(false);
+        stage(false);                            // (unconditional, as in the forward)
+        if (writes && t0 + st < Tlen) {          // (after stage(), which waits for everything outstanding: see the forward)
+            const size_t o = base + (size_t)(t0 + st) * C + sc;
+            store4(gr + o, a4);
+            store4(qbuf + o, b4);
+        }
         __syncthreads();
     }
 
@@ -395,7 +403,7 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
     stage(true);
     __syncthreads();
     for (int t0 = last0; t0 >= 0; t0 -= CH) {
-        if (t0 - CH >= 0) fetch(t0 - CH, true);
+        fetch(t0 - CH, true);                    // (before the start: a clamped fetch that nobody stages)
         const int nt = min(CH, Tlen - t0);
         {
             const int tf = nt - 1;
@@ -459,22 +467,22 @@ __global__ __launch_bounds__(NT, EL == 8 ? 4 : 2) void rec_backward(int Tlen, in
             A += (t0q + t1) + (t2 + t3);
         }
         __syncthreads();
+        float a4[4], b4[4], c4[4];
         if (writes) {
-            float a4[4], b4[4], c4[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 a4[e] = p_a[st][0][wl + e];
                 c4[e] = p_a[st][1][wl + e];
                 b4[e] = fmaf(s_g[st][sc + e], s_rho[st], sum4(p_b, st, wl + e));
             }
-            if (t0 + st < Tlen) {
-                const size_t o = base + (size_t)(t0 + st) * C + sc;
-                store4(gk + o, a4);
-                store4(gv + o, b4);
-                if (PER_TOKEN_W) store4(gw_tok + o, c4);
-            }
         }
-        if (t0 - CH >= 0) stage(true);           // no barrier needed, as in sweep 1
+        stage(true);                             // no barrier needed, as in sweep 1; unconditional, as in the forward
+        if (writes && t0 + st < Tlen) {          // (after stage(), as in sweep 1)
+            const size_t o = base + (size_t)(t0 + st) * C + sc;
+            store4(gk + o, a4);
+            store4(gv + o, b4);
+            if (PER_TOKEN_W) store4(gw_tok + o, c4);
+        }
         __syncthreads();
     }
 
