@@ -146,7 +146,7 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         const float *__restrict__ time_first, const T *__restrict__ k, const T *__restrict__ v,
         const float *__restrict__ s_in, T *__restrict__ y, float *__restrict__ s_out, float *__restrict__ ckpt)
 {
-    __shared__ float start_all[V4_GROUPS][2 * V4_YW][3][64];
+    __shared__ float start_all[V4_GROUPS][2 * V4_YW][5][64];      // the state at a block's start: p, q, o (and dp, dq for the checkpoint)
     // k and v of the blocks of two laps, [token][chain]: left there by the walking wavefront on its way (it is also
     // how the 16-byte pieces reach their owners), read by the wavefront that forms the block's outputs a lap later
     extern __shared__ __align__(16) unsigned char kv_raw[];          // v4_forward_lds<T>() bytes
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
     const int chain_grp = (blockIdx.x * V4_GROUPS + grp) * 64, chain0 = min(chain_grp, (BC - 1) / 64 * 64);
     const int idx = min(chain0 + lane, BC - 1);
     const bool live = chain_grp + lane < BC;
-    float (*start)[3][64] = start_all[grp];
+    float (*start)[5][64] = start_all[grp];
     const int b = idx / C, c = idx % C;
     const float w = -__expf(time_decay[c]), u = time_first[c];
     const size_t base = (size_t)b * Tlen * C + c;
@@ -175,22 +175,31 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         // two laps of blocks: one being consumed, one in flight (named, not an array: every use is a fixed register set)
         static_assert(V4_YW == 3, "the laps are written out for three blocks");
         In k0, k1, k2, k3, k4, k5, v0, v1, v2, v3, v4, v5;
+        // (The 16-byte fetches of the two-byte types are unconditional, also for blocks past the end, where they
+        // repeat the last token and nobody uses them: after a load inside a branch the compiler waits for everything
+        // outstanding instead of for the block it needs.  Measured at B8 T4096 C4096: bf16 forward 265 -> 259 us; fp32,
+        // whose laps in flight are twice the bytes, 316 -> 331 us, so it keeps the conditional fetches.)
+        constexpr bool AHEAD = WIDE && sizeof(T) == 2;
         auto first = [&](int d, In &ik, In &iv) __attribute__((always_inline)) {
-            if (d < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, d * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, d * CK, lane); }
+            if (AHEAD || d < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, d * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, d * CK, lane); }
         };
         first(0, k0, v0); first(1, k1, v1); first(2, k2, v2); first(3, k3, v3); first(4, k4, v4); first(5, k5, v5);
         auto block = [&](int blk, int slot, In &ik, In &iv) __attribute__((always_inline)) {
-            if (blk >= nblk) return;
-            start[slot][0][lane] = s.p; start[slot][1][lane] = s.q; start[slot][2][lane] = s.o;
-            if (ckpt && live) {
-                float *cp = ckpt + (size_t)blk * 5 * BC + idx;
-                cp[0] = s.p; cp[BC] = s.q; cp[2 * (size_t)BC] = s.o; cp[3 * (size_t)BC] = s.dp; cp[4 * (size_t)BC] = s.dq;
-            }
+            if (!AHEAD && blk >= nblk) return;
+            const bool on = blk < nblk;          // scalar
             T kk[CK], vv[CK];
+            if (on) {
+            // (the block's checkpoint is written by the wavefront that forms its outputs, from these five values: this
+            // wavefront then has loads outstanding and nothing else, and loads alone are counted in order, so that a wait
+            // for one block's inputs does not wait for the blocks fetched after it; with a store among them it would)
+            start[slot][0][lane] = s.p; start[slot][1][lane] = s.q; start[slot][2][lane] = s.o;
+            start[slot][3][lane] = s.dp; start[slot][4][lane] = s.dq;
             ik.spread(kv_all[grp][slot][0], lane, kk);
             iv.spread(kv_all[grp][slot][1], lane, vv);
+            }
             const int nb = blk + 2 * V4_YW;
-            if (nb < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, nb * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, nb * CK, lane); }
+            if (AHEAD || nb < nblk) { ik.fetch(k, chain0, idx, BC, C, Tlen, nb * CK, lane); iv.fetch(v, chain0, idx, BC, C, Tlen, nb * CK, lane); }
+            if (!on) return;
             const int t0 = blk * CK, cnt = min(CK, Tlen - t0);
             if (cnt == CK) {
 #pragma unroll
@@ -204,10 +213,8 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         for (int rd = 0; rd <= nlap; rd += 2) {
             block(rd * V4_YW, 0, k0, v0); block(rd * V4_YW + 1, 1, k1, v1); block(rd * V4_YW + 2, 2, k2, v2);
             lds_barrier();
-            if (rd + 1 <= nlap) {
-                block((rd + 1) * V4_YW, 3, k3, v3); block((rd + 1) * V4_YW + 1, 4, k4, v4); block((rd + 1) * V4_YW + 2, 5, k5, v5);
-                lds_barrier();
-            }
+            block((rd + 1) * V4_YW, 3, k3, v3); block((rd + 1) * V4_YW + 1, 4, k4, v4); block((rd + 1) * V4_YW + 2, 5, k5, v5);
+            lds_barrier();                       // (both halves always: blocks past the end do nothing)
         }
         if (s_out && live) { s_out[idx * 3] = s.p; s_out[idx * 3 + 1] = s.q; s_out[idx * 3 + 2] = s.o; }
     } else {
@@ -215,7 +222,13 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         // the outputs of this wavefront's block of lap pr (whose starting state and inputs wait in slot `slot`)
         auto outputs = [&](int pr, int slot) __attribute__((always_inline)) {
             const int blk = pr * V4_YW + r;
-            if (!y || pr < 0 || blk >= nblk) return;
+            if (pr < 0 || blk >= nblk) return;
+            if (ckpt && live) {
+                float *cp = ckpt + (size_t)blk * 5 * BC + idx;
+                cp[0] = start[slot][0][lane]; cp[BC] = start[slot][1][lane]; cp[2 * (size_t)BC] = start[slot][2][lane];
+                cp[3 * (size_t)BC] = start[slot][3][lane]; cp[4 * (size_t)BC] = start[slot][4][lane];
+            }
+            if (!y) return;
             Chain s{start[slot][0][lane], start[slot][1][lane], start[slot][2][lane], 0.f, 0.f};
             const T *ks = kv_all[grp][slot][0], *vs = kv_all[grp][slot][1];
             T kk[CK], vv[CK];
@@ -243,10 +256,8 @@ __global__ __launch_bounds__(64 * (1 + V4_YW) * V4_GROUPS) void v4_forward(int B
         for (int rd = 0; rd <= nlap; rd += 2) {       // in lap rd: the block of lap rd-1
             outputs(rd - 1, V4_YW + r);
             lds_barrier();
-            if (rd + 1 <= nlap) {
-                outputs(rd, r);
-                lds_barrier();
-            }
+            outputs(rd, r);
+            lds_barrier();
         }
     }
 }
