@@ -68,12 +68,12 @@ def test_recurrent_matches_oracle(version, dtype, T):
 
 @pytest.mark.parametrize("version", [5, 6])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-@pytest.mark.parametrize("B,T", [(8, 40), (4, 33)])
+@pytest.mark.parametrize("B,T", [(8, 40), (4, 33), (4, 1), (4, 16)])
 def test_recurrent_with_many_heads(version, dtype, B, T):
     """The per-token kernels pick their form by how the heads fill the compute units: B*H = 512 (twice the 256 compute
     units of an MI355X) and 256 (once) take one workgroup per head with sixteen state elements per lane, where the
     small shapes of the other tests take two workgroups per head with eight.  T = 40 and 33: whole and ragged blocks
-    of sixteen staged tokens, and a last block of one."""
+    of sixteen staged tokens, and a last block of one; T = 1 and 16: a single token, a single whole block."""
     from rwkv_wkv_hip import configs
     wl = configs.make(1 if version == 5 else 3, seed=5, B=B, T=T, C=4096, H=64, dtype=dtype)
     print(f"case v{version} {dtype} B={B} T={T}", flush=True)
