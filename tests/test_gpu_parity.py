@@ -106,9 +106,10 @@ def test_floor_on_decay_and_its_zero_gradient(version):
 
 
 @pytest.mark.parametrize("version", [5, 6])
-def test_no_state_gradient_truncated_bptt(version):
+@pytest.mark.parametrize("B,T,H", [(2, 128, 2), (4, 40, 64)])      # (few heads, many heads: the two forms of the kernels)
+def test_no_state_gradient_truncated_bptt(version, B, T, H):
     from rwkv_wkv_hip import configs
-    wl = configs.make(1 if version == 5 else 3, B=2, T=128, C=128, H=2, dtype=torch.bfloat16)
+    wl = configs.make(1 if version == 5 else 3, B=B, T=T, C=64 * H, H=H, dtype=torch.bfloat16)
     got = run_gpu56(version, wl, with_gstate=False, algo="recurrent")
     ref = run_oracle56(version, wl, with_gstate=False)
     for n in NAMES:
